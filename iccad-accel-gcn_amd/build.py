@@ -1,0 +1,65 @@
+"""Compiles the HIP library for gfx950 in-tree: lib/libaccelgcn.so.
+
+hipcc cross-compiles without a GPU.  Packed-FP32 instruction selection is
+switched off for the device code (scalar fp32 FMAs are used instead).
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent
+ROOT = PKG.parent
+CSRC = PKG / "csrc"
+LIB_DIR = PKG / "lib"
+LIB = LIB_DIR / "libaccelgcn.so"
+SOURCES = ["capi.hip", "preprocess.hip", "spmm.hip", "spmm_accel.cpp"]
+ARCH = "gfx950"
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not Path(exe).exists():
+        raise RuntimeError("hipcc not found; the library cannot be built")
+    return exe
+
+
+def compile_flags():
+    return ["-x", "hip", f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC",
+            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+            "-Wall", "-Wno-unused-command-line-argument",
+            f"-I{ROOT / 'include'}", f"-I{CSRC}"]
+
+
+def build(verbose: bool = False, extra_flags=()) -> Path:
+    LIB_DIR.mkdir(exist_ok=True)
+    objs = []
+    procs = []
+    for src in SOURCES:
+        obj = LIB_DIR / (src + ".o")
+        cmd = [hipcc(), *compile_flags(), *extra_flags, "-c", str(CSRC / src), "-o", str(obj)]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(str(obj))
+    failed = []
+    for src, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            failed.append((src, out))
+        elif verbose and out.strip():
+            print(out)
+    if failed:
+        raise RuntimeError("hipcc failed:\n" + "\n".join(f"--- {s}\n{o}" for s, o in failed))
+    tmp = LIB.with_suffix(".so.tmp")
+    cmd = [hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", str(tmp)]
+    subprocess.run(cmd, check=True)
+    os.replace(tmp, LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose="-v" in sys.argv))

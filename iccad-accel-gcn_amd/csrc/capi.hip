@@ -1,0 +1,529 @@
+// extern "C" surface of the library (declared in include/accel_gcn.h).
+#include <algorithm>
+#include <cstring>
+#include <fstream>
+#include <new>
+#include <vector>
+
+#include "internal.h"
+
+namespace accel {
+
+static thread_local std::string g_error;
+
+void set_error(const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_error = buf;
+}
+const char *get_error() { return g_error.c_str(); }
+void clear_error() { g_error.clear(); }
+
+int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
+                          int32_t **block4_dev, int64_t *n_blocks);
+
+static void release_products(accel_handle *h)
+{
+    if (h->perm) (void)hipFree(h->perm);
+    if (h->s_indptr) (void)hipFree(h->s_indptr);
+    if (h->owns_sorted) {
+        if (h->s_idx) (void)hipFree(const_cast<int32_t *>(h->s_idx));
+        if (h->s_val) (void)hipFree(const_cast<float *>(h->s_val));
+    }
+    if (h->row_block) (void)hipFree(h->row_block);
+    if (h->block4) (void)hipFree(h->block4);
+    if (h->partial) (void)hipFree(h->partial);
+    h->perm = nullptr; h->s_indptr = nullptr; h->s_idx = nullptr; h->s_val = nullptr;
+    h->row_block = nullptr; h->block4 = nullptr; h->partial = nullptr;
+    h->partial_floats = 0; h->owns_sorted = false; h->ready = false;
+}
+
+static int need_gpu()
+{
+    int n = 0;
+    const hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        set_error("no HIP device available (%s); this library has no CPU fallback",
+                  e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+        return ACCEL_ERR_HIP;
+    }
+    return ACCEL_OK;
+}
+
+}  // namespace accel
+
+using namespace accel;
+
+extern "C" {
+
+const char *accel_last_error(void) { return get_error(); }
+int accel_version(void) { return 100; }
+
+// ---------------------------------------------------------------------------
+// host utilities
+// ---------------------------------------------------------------------------
+int accel_partition_host(const int32_t *indptr, int64_t rows, int32_t *block4_out, int64_t cap,
+                         int64_t *n_blocks)
+{
+    clear_error();
+    if (!indptr || rows < 0 || !n_blocks || cap < 0 || (cap > 0 && !block4_out)) {
+        set_error("accel_partition_host: bad argument");
+        return ACCEL_ERR_ARG;
+    }
+    if (indptr[0] != 0) {
+        set_error("indptr must start at 0");
+        return ACCEL_ERR_CSR;
+    }
+    int64_t nb = 0;
+    auto put = [&](int d, int64_t row, int64_t loc, int info) {
+        if (nb < cap) {
+            int32_t *q = block4_out + 4 * nb;
+            q[0] = d; q[1] = (int32_t)row; q[2] = (int32_t)loc; q[3] = info;
+        }
+        nb++;
+    };
+    // one pass over maximal runs of equal degree
+    int64_t r = 0;
+    while (r < rows) {
+        const int64_t d64 = (int64_t)indptr[r + 1] - indptr[r];
+        if (d64 < 0) {
+            set_error("indptr decreases at row %lld", (long long)r);
+            return ACCEL_ERR_CSR;
+        }
+        int64_t end = r + 1;
+        while (end < rows && (int64_t)indptr[end + 1] - indptr[end] == d64) end++;
+        const int d = (int)d64;
+        if (d > kDegBound) {
+            for (int64_t q = r; q < end; q++)
+                for (int off = 0; off < d; off += kDegBound)
+                    put(d, q, (int64_t)indptr[q] + off, std::min(kDegBound, d - off));
+        } else if (d > 0) {
+            int w, rpb;
+            slice_rule(d, w, rpb);
+            for (int64_t q = r; q < end; q += rpb)
+                put(d, q, indptr[q], (w << 16) + (int)std::min<int64_t>(rpb, end - q));
+        }
+        r = end;
+    }
+    *n_blocks = nb;
+    return ACCEL_OK;
+}
+
+int accel_degree_sort_host(const int32_t *indptr, int64_t rows, int32_t *perm_out)
+{
+    clear_error();
+    if (!indptr || rows < 0 || (rows > 0 && !perm_out)) {
+        set_error("accel_degree_sort_host: bad argument");
+        return ACCEL_ERR_ARG;
+    }
+    std::vector<uint64_t> keys;
+    try {
+        keys.resize((size_t)rows);
+    } catch (const std::bad_alloc &) {
+        set_error("host allocation failed");
+        return ACCEL_ERR_ALLOC;
+    }
+    for (int64_t r = 0; r < rows; r++) {
+        const int64_t d = (int64_t)indptr[r + 1] - indptr[r];
+        if (d < 0) {
+            set_error("indptr decreases at row %lld", (long long)r);
+            return ACCEL_ERR_CSR;
+        }
+        keys[(size_t)r] = ((uint64_t)d << 32) | (uint64_t)r;   // unique keys: any sort is stable
+    }
+    std::sort(keys.begin(), keys.end());
+    for (int64_t r = 0; r < rows; r++) perm_out[r] = (int32_t)(keys[(size_t)r] & 0xFFFFFFFFu);
+    return ACCEL_OK;
+}
+
+// ---------------------------------------------------------------------------
+// raw-array files
+// ---------------------------------------------------------------------------
+int accel_file_count(const char *path, int64_t *n_elems)
+{
+    clear_error();
+    if (!path || !n_elems) { set_error("accel_file_count: bad argument"); return ACCEL_ERR_ARG; }
+    std::ifstream f(path, std::ios::binary | std::ios::ate);
+    if (!f) { set_error("cannot open %s", path); return ACCEL_ERR_IO; }
+    const std::streamoff len = f.tellg();
+    if (len < 0 || len % 4 != 0) {
+        set_error("%s: size %lld is not a whole number of 4-byte elements", path, (long long)len);
+        return ACCEL_ERR_IO;
+    }
+    *n_elems = (int64_t)(len / 4);
+    return ACCEL_OK;
+}
+
+int accel_file_read(const char *path, void *dst, int64_t n_elems)
+{
+    clear_error();
+    if (!path || n_elems < 0 || (n_elems > 0 && !dst)) {
+        set_error("accel_file_read: bad argument");
+        return ACCEL_ERR_ARG;
+    }
+    std::ifstream f(path, std::ios::binary);
+    if (!f) { set_error("cannot open %s", path); return ACCEL_ERR_IO; }
+    f.read(static_cast<char *>(dst), (std::streamsize)(n_elems * 4));
+    if (f.gcount() != (std::streamsize)(n_elems * 4)) {
+        set_error("%s: short read (%lld of %lld bytes)", path, (long long)f.gcount(),
+                  (long long)(n_elems * 4));
+        return ACCEL_ERR_IO;
+    }
+    return ACCEL_OK;
+}
+
+int accel_file_write(const char *path, const void *src, int64_t n_elems)
+{
+    clear_error();
+    if (!path || n_elems < 0 || (n_elems > 0 && !src)) {
+        set_error("accel_file_write: bad argument");
+        return ACCEL_ERR_ARG;
+    }
+    std::ofstream f(path, std::ios::binary | std::ios::trunc);
+    if (!f) { set_error("cannot create %s", path); return ACCEL_ERR_IO; }
+    f.write(static_cast<const char *>(src), (std::streamsize)(n_elems * 4));
+    f.close();
+    if (!f) { set_error("write to %s failed", path); return ACCEL_ERR_IO; }
+    return ACCEL_OK;
+}
+
+// ---------------------------------------------------------------------------
+// device plumbing
+// ---------------------------------------------------------------------------
+int accel_device_count(int *n)
+{
+    clear_error();
+    if (!n) { set_error("accel_device_count: null argument"); return ACCEL_ERR_ARG; }
+    *n = 0;
+    const hipError_t e = hipGetDeviceCount(n);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *n = 0;
+        set_error("hipGetDeviceCount: %s", hipGetErrorString(e));
+        return ACCEL_ERR_HIP;
+    }
+    return ACCEL_OK;
+}
+
+int accel_dev_malloc(void **p, size_t bytes)
+{
+    clear_error();
+    if (!p) { set_error("accel_dev_malloc: null argument"); return ACCEL_ERR_ARG; }
+    *p = nullptr;
+    if (int rc = need_gpu()) return rc;
+    if (hipMalloc(p, bytes ? bytes : 4) != hipSuccess) {
+        (void)hipGetLastError();
+        *p = nullptr;
+        set_error("device allocation of %zu bytes failed", bytes);
+        return ACCEL_ERR_ALLOC;
+    }
+    return ACCEL_OK;
+}
+
+int accel_dev_free(void *p)
+{
+    clear_error();
+    if (p) ACCEL_HIP(hipFree(p));
+    return ACCEL_OK;
+}
+
+int accel_memcpy_h2d(void *dst, const void *src, size_t bytes)
+{
+    clear_error();
+    if (bytes && (!dst || !src)) { set_error("accel_memcpy_h2d: null argument"); return ACCEL_ERR_ARG; }
+    if (bytes) ACCEL_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return ACCEL_OK;
+}
+
+int accel_memcpy_d2h(void *dst, const void *src, size_t bytes)
+{
+    clear_error();
+    if (bytes && (!dst || !src)) { set_error("accel_memcpy_d2h: null argument"); return ACCEL_ERR_ARG; }
+    if (bytes) ACCEL_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return ACCEL_OK;
+}
+
+int accel_dev_fill_u32(void *dst, uint32_t value, size_t n_words, void *stream)
+{
+    clear_error();
+    if (n_words && !dst) { set_error("accel_dev_fill_u32: null argument"); return ACCEL_ERR_ARG; }
+    return fill_u32(dst, value, n_words, static_cast<hipStream_t>(stream));
+}
+
+int accel_stream_sync(void *stream)
+{
+    clear_error();
+    ACCEL_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return ACCEL_OK;
+}
+
+// ---------------------------------------------------------------------------
+// operator
+// ---------------------------------------------------------------------------
+int accel_create(const int32_t *indptr, const int32_t *idx, const float *val, int64_t rows,
+                 int64_t cols, int64_t nnz, int flags, accel_handle **out)
+{
+    clear_error();
+    if (!out) { set_error("accel_create: null handle pointer"); return ACCEL_ERR_ARG; }
+    *out = nullptr;
+    if (rows < 0 || cols < 0 || nnz < 0 || rows >= 0x7fffffffLL || cols > 0x7fffffffLL ||
+        nnz > 0x7fffffffLL) {
+        set_error("accel_create: rows/cols/nnz must be non-negative and fit int32");
+        return ACCEL_ERR_ARG;
+    }
+    if (!indptr || (nnz > 0 && (!idx || !val))) {
+        set_error("accel_create: null CSR array");
+        return ACCEL_ERR_ARG;
+    }
+    if (flags != ACCEL_PTR_HOST && flags != ACCEL_PTR_DEVICE) {
+        set_error("accel_create: unknown flags %d", flags);
+        return ACCEL_ERR_ARG;
+    }
+    if (int rc = need_gpu()) return rc;
+    accel_handle *h = new (std::nothrow) accel_handle();
+    if (!h) { set_error("host allocation failed"); return ACCEL_ERR_ALLOC; }
+    h->rows = rows; h->cols = cols; h->nnz = nnz;
+    (void)hipGetDevice(&h->device);
+    if (flags == ACCEL_PTR_DEVICE) {
+        h->indptr = indptr; h->idx = idx; h->val = val;
+        h->owns_input = false;
+    } else {
+        void *a = nullptr, *b = nullptr, *c = nullptr;
+        const size_t sa = sizeof(int32_t) * (size_t)(rows + 1);
+        const size_t sb = sizeof(int32_t) * (size_t)nnz, sc = sizeof(float) * (size_t)nnz;
+        if (hipMalloc(&a, sa) != hipSuccess || hipMalloc(&b, sb ? sb : 4) != hipSuccess ||
+            hipMalloc(&c, sc ? sc : 4) != hipSuccess) {
+            (void)hipGetLastError();
+            if (a) (void)hipFree(a);
+            if (b) (void)hipFree(b);
+            if (c) (void)hipFree(c);
+            delete h;
+            set_error("device allocation for the CSR (%zu bytes) failed", sa + sb + sc);
+            return ACCEL_ERR_ALLOC;
+        }
+        h->indptr = static_cast<int32_t *>(a);
+        h->idx = static_cast<int32_t *>(b);
+        h->val = static_cast<float *>(c);
+        h->owns_input = true;
+        hipError_t e = hipMemcpy(a, indptr, sa, hipMemcpyHostToDevice);
+        if (e == hipSuccess && sb) e = hipMemcpy(b, idx, sb, hipMemcpyHostToDevice);
+        if (e == hipSuccess && sc) e = hipMemcpy(c, val, sc, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            set_error("upload of the CSR failed: %s", hipGetErrorString(e));
+            accel_destroy(h);
+            return ACCEL_ERR_HIP;
+        }
+    }
+    *out = h;
+    return ACCEL_OK;
+}
+
+int accel_destroy(accel_handle *h)
+{
+    if (!h) return ACCEL_OK;
+    release_products(h);
+    if (h->owns_input) {
+        (void)hipFree(const_cast<int32_t *>(h->indptr));
+        (void)hipFree(const_cast<int32_t *>(h->idx));
+        (void)hipFree(const_cast<float *>(h->val));
+    }
+    delete h;
+    return ACCEL_OK;
+}
+
+int accel_preprocess(accel_handle *h)
+{
+    clear_error();
+    if (!h) { set_error("accel_preprocess: null handle"); return ACCEL_ERR_ARG; }
+    release_products(h);
+    const int rc = preprocess_device(h);
+    if (rc) release_products(h);
+    return rc;
+}
+
+int accel_get_info(const accel_handle *h, accel_info *out)
+{
+    clear_error();
+    if (!h || !out) { set_error("accel_get_info: null argument"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_get_info: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    out->rows = h->rows; out->cols = h->cols; out->nnz = h->nnz;
+    out->n_blocks = h->n_blocks; out->n_long_blocks = h->n_long_blocks;
+    out->n_long_rows = h->n_long_rows; out->n_zero_rows = h->n_zero_rows;
+    out->max_degree = h->max_degree; out->already_sorted = h->identity_perm ? 1 : 0;
+    out->preprocess_ms = h->preprocess_ms;
+    return ACCEL_OK;
+}
+
+int accel_get_block4(const accel_handle *h, int32_t *out, int64_t cap_blocks)
+{
+    clear_error();
+    if (!h || (!out && h->n_blocks > 0)) { set_error("accel_get_block4: null argument"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_get_block4: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (cap_blocks < h->n_blocks) {
+        set_error("accel_get_block4: buffer holds %lld blocks, %lld needed", (long long)cap_blocks,
+                  (long long)h->n_blocks);
+        return ACCEL_ERR_ARG;
+    }
+    if (h->n_blocks)
+        ACCEL_HIP(hipMemcpy(out, h->block4, sizeof(int32_t) * 4 * (size_t)h->n_blocks,
+                            hipMemcpyDeviceToHost));
+    return ACCEL_OK;
+}
+
+int accel_get_perm(const accel_handle *h, int32_t *out, int64_t cap_rows)
+{
+    clear_error();
+    if (!h || (!out && h->rows > 0)) { set_error("accel_get_perm: null argument"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_get_perm: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (cap_rows < h->rows) { set_error("accel_get_perm: buffer too small"); return ACCEL_ERR_ARG; }
+    if (h->identity_perm) {
+        for (int64_t r = 0; r < h->rows; r++) out[r] = (int32_t)r;
+    } else {
+        ACCEL_HIP(hipMemcpy(out, h->perm, sizeof(int32_t) * (size_t)h->rows, hipMemcpyDeviceToHost));
+    }
+    return ACCEL_OK;
+}
+
+int accel_get_sorted_csr(const accel_handle *h, int32_t *indptr, int32_t *idx, float *val)
+{
+    clear_error();
+    if (!h) { set_error("accel_get_sorted_csr: null handle"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_get_sorted_csr: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (h->rows == 0) {
+        if (indptr) indptr[0] = 0;
+        return ACCEL_OK;
+    }
+    if (indptr)
+        ACCEL_HIP(hipMemcpy(indptr, h->s_indptr, sizeof(int32_t) * (size_t)(h->rows + 1),
+                            hipMemcpyDeviceToHost));
+    if (idx && h->nnz)
+        ACCEL_HIP(hipMemcpy(idx, h->s_idx, sizeof(int32_t) * (size_t)h->nnz, hipMemcpyDeviceToHost));
+    if (val && h->nnz)
+        ACCEL_HIP(hipMemcpy(val, h->s_val, sizeof(float) * (size_t)h->nnz, hipMemcpyDeviceToHost));
+    return ACCEL_OK;
+}
+
+int accel_check_block4(accel_handle *h, const int32_t *block4_host, int64_t n_blocks)
+{
+    clear_error();
+    if (!h || n_blocks < 0 || (n_blocks > 0 && !block4_host)) {
+        set_error("accel_check_block4: bad argument");
+        return ACCEL_ERR_ARG;
+    }
+    if (!h->ready) { set_error("accel_check_block4: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (n_blocks != h->n_blocks) {
+        set_error("metadata has %lld blocks, this CSR partitions into %lld", (long long)n_blocks,
+                  (long long)h->n_blocks);
+        return ACCEL_ERR_META;
+    }
+    std::vector<int32_t> mine((size_t)n_blocks * 4);
+    if (n_blocks)
+        ACCEL_HIP(hipMemcpy(mine.data(), h->block4, sizeof(int32_t) * mine.size(), hipMemcpyDeviceToHost));
+    for (size_t i = 0; i < mine.size(); i++)
+        if (mine[i] != block4_host[i]) {
+            set_error("metadata differs at block %zu field %zu: file %d, CSR %d", i / 4, i % 4,
+                      block4_host[i], mine[i]);
+            return ACCEL_ERR_META;
+        }
+    return ACCEL_OK;
+}
+
+// Partition a row order as given, on the GPU: what block_level_partition.py
+// computes for one *.new_indptr file (lines 38-106).  indptr is a host array.
+int accel_partition_gpu(const int32_t *indptr, int64_t rows, int32_t *block4_out, int64_t cap,
+                        int64_t *n_blocks)
+{
+    clear_error();
+    if (!indptr || rows < 0 || rows >= 0x7fffffffLL || !n_blocks || cap < 0 ||
+        (cap > 0 && !block4_out)) {
+        set_error("accel_partition_gpu: bad argument");
+        return ACCEL_ERR_ARG;
+    }
+    if (int rc = need_gpu()) return rc;
+    *n_blocks = 0;
+    if (rows == 0) return ACCEL_OK;
+    void *dptr = nullptr;
+    if (hipMalloc(&dptr, sizeof(int32_t) * (size_t)(rows + 1)) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("device allocation failed");
+        return ACCEL_ERR_ALLOC;
+    }
+    int rc = ACCEL_OK;
+    int32_t *b4 = nullptr;
+    int64_t nb = 0;
+    if (hipMemcpy(dptr, indptr, sizeof(int32_t) * (size_t)(rows + 1), hipMemcpyHostToDevice) != hipSuccess) {
+        set_error("upload of indptr failed");
+        rc = ACCEL_ERR_HIP;
+    }
+    if (!rc) rc = partition_only_device(static_cast<int32_t *>(dptr), rows, indptr[rows], &b4, &nb);
+    if (!rc) {
+        *n_blocks = nb;
+        const int64_t take = std::min(nb, cap);
+        if (take > 0 &&
+            hipMemcpy(block4_out, b4, sizeof(int32_t) * 4 * (size_t)take, hipMemcpyDeviceToHost) != hipSuccess) {
+            set_error("download of the metadata failed");
+            rc = ACCEL_ERR_HIP;
+        }
+    }
+    if (b4) (void)hipFree(b4);
+    (void)hipFree(dptr);
+    return rc;
+}
+
+int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream)
+{
+    clear_error();
+    if (!h) { set_error("accel_run: null handle"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_run: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (N <= 0) { set_error("accel_run: N must be positive, got %d", N); return ACCEL_ERR_ARG; }
+    if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("accel_run: null dense operand"); return ACCEL_ERR_ARG; }
+    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr);
+}
+
+int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup, int iters,
+               float *ms_total, float *ms_main, void *stream)
+{
+    clear_error();
+    if (!h) { set_error("accel_time: null handle"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_time: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (N <= 0 || warmup < 0 || iters < 0) { set_error("accel_time: bad N/warmup/iters"); return ACCEL_ERR_ARG; }
+    if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("accel_time: null dense operand"); return ACCEL_ERR_ARG; }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (int i = 0; i < warmup; i++)
+        if (int rc = spmm_launch(h, X, Y, N, s, nullptr)) return rc;
+    ACCEL_HIP(hipStreamSynchronize(s));
+    hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr;
+    ACCEL_HIP(hipEventCreate(&e0));
+    ACCEL_HIP(hipEventCreate(&e1));
+    ACCEL_HIP(hipEventCreate(&e2));
+    int rc = ACCEL_OK;
+    for (int i = 0; i < iters && !rc; i++) {
+        hipError_t e = hipEventRecord(e0, s);
+        if (e == hipSuccess) rc = spmm_launch(h, X, Y, N, s, ms_main ? e1 : nullptr);
+        if (rc) break;
+        if (e == hipSuccess) e = hipEventRecord(e2, s);
+        if (e == hipSuccess) e = hipEventSynchronize(e2);
+        float t = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&t, e0, e2);
+        if (e == hipSuccess && ms_total) ms_total[i] = t;
+        if (e == hipSuccess && ms_main) {
+            e = hipEventElapsedTime(&t, e0, e1);
+            ms_main[i] = t;
+        }
+        if (e != hipSuccess) {
+            set_error("event timing failed: %s", hipGetErrorString(e));
+            rc = ACCEL_ERR_HIP;
+        }
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipEventDestroy(e2);
+    return rc;
+}
+
+}  // extern "C"

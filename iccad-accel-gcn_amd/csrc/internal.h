@@ -1,0 +1,79 @@
+// Shared declarations of the library's translation units (not installed).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "accel_gcn.h"
+
+namespace accel {
+
+constexpr int kDegBound = ACCEL_DEG_BOUND;            // non-zeros per block4 entry
+constexpr int kSlices = ACCEL_SLICES_PER_BLOCK;       // slices per entry (metadata ABI)
+constexpr int kSliceNz = kDegBound / kSlices;         // 32
+
+// last-error string of the calling thread
+void set_error(const char *fmt, ...);
+const char *get_error();
+void clear_error();
+
+#define ACCEL_HIP(call)                                                                     \
+    do {                                                                                    \
+        hipError_t e_ = (call);                                                             \
+        if (e_ != hipSuccess) {                                                             \
+            accel::set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_),         \
+                             __FILE__, __LINE__);                                           \
+            return ACCEL_ERR_HIP;                                                           \
+        }                                                                                   \
+    } while (0)
+
+// Slice rule of the block4 metadata for a row degree 1..384
+// (block_level_partition.py:12-21 tables, :56-63 defaults beyond the table).
+__host__ __device__ inline void slice_rule(int d, int &w_nz, int &rows_per_block)
+{
+    if (d >= kDegBound / 2) { w_nz = kSliceNz; rows_per_block = 1; return; }
+    const int split = d <= 32 ? 1 : d <= 64 ? 2 : d <= 96 ? 3 : d <= 128 ? 4 : 6;
+    w_nz = (d + split - 1) / split;
+    rows_per_block = kSlices / split;
+}
+
+}  // namespace accel
+
+// The operator state behind the opaque C handle.
+struct accel_handle {
+    int64_t rows = 0, cols = 0, nnz = 0;
+    int device = 0;
+    // caller's CSR on the device (owned when uploaded from the host)
+    const int32_t *indptr = nullptr;
+    const int32_t *idx = nullptr;
+    const float *val = nullptr;
+    bool owns_input = false;
+    // preprocess products
+    bool ready = false;
+    bool identity_perm = false;       // input already degree-sorted: perm == iota
+    int32_t *perm = nullptr;          // [rows] new row -> caller's row (nullptr when identity)
+    int32_t *s_indptr = nullptr;      // [rows+1] degree-sorted CSR
+    const int32_t *s_idx = nullptr;   // [nnz]  (aliases idx when identity)
+    const float *s_val = nullptr;     // [nnz]  (aliases val when identity)
+    bool owns_sorted = false;
+    int32_t *row_block = nullptr;     // [rows+1] first block4 entry of each sorted row
+    int32_t *block4 = nullptr;        // [4*n_blocks]
+    int64_t n_blocks = 0, n_long_blocks = 0, n_long_rows = 0, n_zero_rows = 0;
+    int32_t max_degree = 0;
+    double preprocess_ms = 0.0;
+    // scratch for the partial sums of long-row segments: [n_long_blocks * N]
+    float *partial = nullptr;
+    size_t partial_floats = 0;
+};
+
+namespace accel {
+// preprocess.hip
+int preprocess_device(accel_handle *h);
+// spmm.hip
+int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
+                hipEvent_t after_main);
+int fill_u32(void *dst, uint32_t v, size_t n, hipStream_t s);
+}  // namespace accel

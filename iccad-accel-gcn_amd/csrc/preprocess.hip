@@ -1,0 +1,565 @@
+// GPU preprocessing for the SpMM operator: CSR validation, stable degree sort,
+// permuted-CSR gather and the block4 partition metadata.  Integer, HBM-bound
+// work; every kernel is a streaming pass over rows or non-zeros.
+//
+// The metadata rules are those of upstream's block_level_partition.py:7-21
+// (tables) and :48-103 (walk); the walk is restated as a closed form per row so
+// that it runs as scans + one emit kernel:
+//   - a row of degree d in 1..384 that sits (r - s) rows into its maximal run of
+//     equal-degree rows (run start s) opens a block iff (r - s) % rows[d] == 0;
+//     the block takes up to rows[d] rows of that run;
+//   - a row of degree d > 384 opens ceil(d / 384) blocks;
+//   - rows of degree 0 open none.
+#include <algorithm>
+#include <chrono>
+#include <climits>
+#include <vector>
+
+#include "internal.h"
+
+namespace accel {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kItems = 8;
+constexpr int kTile = kThreads * kItems;  // elements per workgroup in scans and sort passes
+
+struct SumOp {
+    static constexpr int identity = 0;
+    __device__ int operator()(int a, int b) const { return a + b; }
+};
+struct MaxOp {
+    static constexpr int identity = INT_MIN;
+    __device__ int operator()(int a, int b) const { return a > b ? a : b; }
+};
+
+// Exclusive scan of one value per thread over a 256-thread workgroup.
+template <class Op>
+__device__ int block_exclusive_scan(int v, Op op, int *wave_tot /* LDS, 4 ints */, int &total)
+{
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    int inc = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int t = __shfl_up(inc, off);
+        if (lane >= off) inc = op(t, inc);
+    }
+    if (lane == 63) wave_tot[w] = inc;
+    __syncthreads();
+    int prefix = Op::identity, tot = Op::identity;
+#pragma unroll
+    for (int i = 0; i < kThreads / 64; i++) {
+        const int t = wave_tot[i];
+        if (i < w) prefix = op(prefix, t);
+        tot = op(tot, t);
+    }
+    __syncthreads();
+    int exc = __shfl_up(inc, 1);
+    if (lane == 0) exc = Op::identity;
+    total = tot;
+    return op(prefix, exc);
+}
+
+template <class Op>
+__global__ __launch_bounds__(kThreads) void scan_reduce(const int *__restrict__ in, int64_t n,
+                                                        int *__restrict__ sums)
+{
+    __shared__ int wave_tot[kThreads / 64];
+    Op op;
+    const int64_t base = (int64_t)blockIdx.x * kTile + (int64_t)threadIdx.x * kItems;
+    int acc = Op::identity;
+#pragma unroll
+    for (int j = 0; j < kItems; j++)
+        if (base + j < n) acc = op(acc, in[base + j]);
+    int total;
+    block_exclusive_scan(acc, op, wave_tot, total);
+    if (threadIdx.x == 0) sums[blockIdx.x] = total;
+}
+
+// One workgroup turns sums[0..nb) into their exclusive scan and stores the grand
+// total at sums[nb].
+template <class Op>
+__global__ __launch_bounds__(kThreads) void scan_spine(int *__restrict__ sums, int64_t nb)
+{
+    __shared__ int wave_tot[kThreads / 64];
+    Op op;
+    int carry = Op::identity;
+    for (int64_t base = 0; base < nb; base += kThreads) {
+        const int64_t i = base + threadIdx.x;
+        const int v = i < nb ? sums[i] : Op::identity;
+        int total;
+        const int exc = block_exclusive_scan(v, op, wave_tot, total);
+        if (i < nb) sums[i] = op(carry, exc);
+        carry = op(carry, total);
+    }
+    if (threadIdx.x == 0) sums[nb] = carry;
+}
+
+template <class Op, bool kInclusive>
+__global__ __launch_bounds__(kThreads) void scan_apply(const int *__restrict__ in, int64_t n,
+                                                       const int *__restrict__ sums,
+                                                       int *__restrict__ out,
+                                                       int *__restrict__ total_out, int64_t nb)
+{
+    __shared__ int wave_tot[kThreads / 64];
+    Op op;
+    const int64_t base = (int64_t)blockIdx.x * kTile + (int64_t)threadIdx.x * kItems;
+    int v[kItems];
+    int acc = Op::identity;
+#pragma unroll
+    for (int j = 0; j < kItems; j++) {
+        v[j] = base + j < n ? in[base + j] : Op::identity;
+        acc = op(acc, v[j]);
+    }
+    int total;
+    int run = op(sums[blockIdx.x], block_exclusive_scan(acc, op, wave_tot, total));
+#pragma unroll
+    for (int j = 0; j < kItems; j++) {
+        const int inc = op(run, v[j]);
+        if (base + j < n) out[base + j] = kInclusive ? inc : run;
+        run = inc;
+    }
+    if (total_out && blockIdx.x == 0 && threadIdx.x == 0) *total_out = sums[nb];
+}
+
+// out = scan(in) over n ints (in place allowed); *total_out (device, optional)
+// receives the reduction of all n.  `sums` needs n/kTile + 2 ints.
+template <class Op, bool kInclusive>
+int device_scan(const int *in, int64_t n, int *out, int *total_out, int *sums, hipStream_t s)
+{
+    if (n <= 0) {
+        if (total_out) return fill_u32(total_out, (uint32_t)Op::identity, 1, s);
+        return ACCEL_OK;
+    }
+    const int64_t nb = (n + kTile - 1) / kTile;
+    scan_reduce<Op><<<dim3((unsigned)nb), dim3(kThreads), 0, s>>>(in, n, sums);
+    scan_spine<Op><<<dim3(1), dim3(kThreads), 0, s>>>(sums, nb);
+    scan_apply<Op, kInclusive><<<dim3((unsigned)nb), dim3(kThreads), 0, s>>>(in, n, sums, out,
+                                                                            total_out, nb);
+    ACCEL_HIP(hipGetLastError());
+    return ACCEL_OK;
+}
+
+// ---------------------------------------------------------------------------
+// CSR validation + degrees
+// ---------------------------------------------------------------------------
+struct Stats {
+    int bad_indptr;     // non-monotone / wrong ends
+    int bad_index;      // column outside [0, cols)
+    int unsorted;       // some row has a smaller degree than its predecessor
+    int max_degree;
+    int n_zero_rows;
+    int n_long_rows;
+    int n_long_blocks;
+};
+
+__global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restrict__ indptr,
+                                                          int64_t rows, int64_t nnz,
+                                                          uint32_t *__restrict__ deg,
+                                                          Stats *__restrict__ st)
+{
+    const int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    int bad = 0, unsorted = 0, d = 0, zero = 0, lrow = 0, lblk = 0;
+    if (r < rows) {
+        const int a = indptr[r], b = indptr[r + 1];
+        d = b - a;
+        if (b < a) { bad = 1; d = 0; }
+        if (r == 0 && a != 0) bad = 1;
+        if (r == rows - 1 && (int64_t)b != nnz) bad = 1;
+        if (r > 0 && !bad) {
+            const int dp = a - indptr[r - 1];
+            if (d < dp) unsorted = 1;
+        }
+        deg[r] = (uint32_t)d;
+        zero = d == 0;
+        if (d > kDegBound) { lrow = 1; lblk = (d + kDegBound - 1) / kDegBound; }
+    }
+    // wave-level combine, one atomic per wave and field
+    const unsigned long long any_bad = __ballot(bad), any_uns = __ballot(unsorted);
+    int m = d;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        m = max(m, __shfl_xor(m, off));
+        lblk += __shfl_xor(lblk, off);
+    }
+    const int nz = __popcll(__ballot(zero)), nl = __popcll(__ballot(lrow));
+    if ((threadIdx.x & 63) == 0) {
+        if (any_bad) atomicOr(&st->bad_indptr, 1);
+        if (any_uns) atomicOr(&st->unsorted, 1);
+        if (m > 0) atomicMax(&st->max_degree, m);
+        if (nz) atomicAdd(&st->n_zero_rows, nz);
+        if (nl) atomicAdd(&st->n_long_rows, nl);
+        if (lblk) atomicAdd(&st->n_long_blocks, lblk);
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void index_check_kernel(const int32_t *__restrict__ idx,
+                                                               int64_t nnz, int64_t cols,
+                                                               Stats *__restrict__ st)
+{
+    int bad = 0;
+    for (int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x; p < nnz;
+         p += (int64_t)gridDim.x * kThreads) {
+        const int c = idx[p];
+        bad |= (c < 0) | ((int64_t)c >= cols);
+    }
+    if (__ballot(bad) && (threadIdx.x & 63) == 0) atomicOr(&st->bad_index, 1);
+}
+
+// ---------------------------------------------------------------------------
+// Stable LSD radix sort of (degree, row) pairs, 8 bits per pass.  Stability is
+// what makes ties keep the caller's row order.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void radix_hist(const uint32_t *__restrict__ keys,
+                                                       int64_t n, int shift,
+                                                       int *__restrict__ hist, int64_t tiles)
+{
+    __shared__ int h[256];
+    h[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * kTile;
+#pragma unroll
+    for (int j = 0; j < kItems; j++) {
+        const int64_t i = base + j * kThreads + threadIdx.x;
+        if (i < n) atomicAdd(&h[(keys[i] >> shift) & 255u], 1);
+    }
+    __syncthreads();
+    hist[(int64_t)threadIdx.x * tiles + blockIdx.x] = h[threadIdx.x];  // digit-major
+}
+
+__global__ __launch_bounds__(kThreads) void radix_scatter(
+    const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
+    uint32_t *__restrict__ keys_out, uint32_t *__restrict__ vals_out, int64_t n, int shift,
+    const int *__restrict__ hist_scanned, int64_t tiles)
+{
+    __shared__ int running[256];               // next output slot of each digit for this tile
+    __shared__ int wave_cnt[kThreads / 64][256];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    running[threadIdx.x] = hist_scanned[(int64_t)threadIdx.x * tiles + blockIdx.x];
+    const int64_t base = (int64_t)blockIdx.x * kTile;
+    for (int j = 0; j < kItems; j++) {
+        const int64_t i = base + j * kThreads + threadIdx.x;
+        const bool valid = i < n;
+        const uint32_t key = valid ? keys_in[i] : 0u;
+        const uint32_t val = valid ? (vals_in ? vals_in[i] : (uint32_t)i) : 0u;
+        const uint32_t dg = (key >> shift) & 255u;
+#pragma unroll
+        for (int q = 0; q < kThreads / 64; q++) wave_cnt[q][threadIdx.x] = 0;
+        __syncthreads();
+        // lanes of this wave that hold the same digit
+        unsigned long long peers = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const bool bit = (dg >> b) & 1u;
+            const unsigned long long bal = __ballot(bit);
+            peers &= bit ? bal : ~bal;
+        }
+        const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+        if (valid && rank == 0) wave_cnt[w][dg] = __popcll(peers);
+        __syncthreads();
+        if (valid) {
+            int pos = running[dg] + rank;
+            for (int q = 0; q < w; q++) pos += wave_cnt[q][dg];
+            keys_out[pos] = key;
+            vals_out[pos] = val;
+        }
+        __syncthreads();
+        int add = 0;
+#pragma unroll
+        for (int q = 0; q < kThreads / 64; q++) add += wave_cnt[q][threadIdx.x];
+        running[threadIdx.x] += add;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void iota_kernel(uint32_t *out, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i < n) out[i] = (uint32_t)i;
+}
+
+// ---------------------------------------------------------------------------
+// Permuted CSR: non-zero p of the sorted matrix comes from the caller's row
+// perm[r], where r is the sorted row that contains p.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void permute_csr_kernel(
+    const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
+    const float *__restrict__ val, const int32_t *__restrict__ perm,
+    const int32_t *__restrict__ s_indptr, int64_t rows, int64_t nnz, int32_t *__restrict__ s_idx,
+    float *__restrict__ s_val)
+{
+    const int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (p >= nnz) return;
+    int64_t lo = 0, hi = rows - 1;  // first row whose end is beyond p
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if ((int64_t)s_indptr[mid + 1] > p) hi = mid; else lo = mid + 1;
+    }
+    const int64_t src = (int64_t)indptr[perm[lo]] + (p - s_indptr[lo]);
+    s_idx[p] = idx[src];
+    s_val[p] = val[src];
+}
+
+// ---------------------------------------------------------------------------
+// Partition
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void run_head_kernel(const uint32_t *__restrict__ deg,
+                                                            int64_t rows, int *__restrict__ head)
+{
+    const int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (r < rows) head[r] = (r == 0 || deg[r] != deg[r - 1]) ? (int)r : 0;
+}
+
+__global__ __launch_bounds__(kThreads) void block_count_kernel(
+    const uint32_t *__restrict__ deg, const int *__restrict__ run_start, int64_t rows,
+    int *__restrict__ count)
+{
+    const int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (r >= rows) return;
+    const int d = (int)deg[r];
+    int c = 0;
+    if (d > kDegBound) {
+        c = (d + kDegBound - 1) / kDegBound;
+    } else if (d > 0) {
+        int w, rpb;
+        slice_rule(d, w, rpb);
+        c = ((int)r - run_start[r]) % rpb == 0;
+    }
+    count[r] = c;
+}
+
+__global__ __launch_bounds__(kThreads) void emit_block4_kernel(
+    const uint32_t *__restrict__ deg, const int32_t *__restrict__ s_indptr,
+    const int *__restrict__ run_start, const int *__restrict__ row_block, int64_t rows,
+    int4 *__restrict__ block4)
+{
+    const int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (r >= rows) return;
+    const int d = (int)deg[r];
+    if (d == 0) return;
+    const int at = row_block[r];
+    const int loc = s_indptr[r];
+    if (d > kDegBound) {
+        const int nseg = (d + kDegBound - 1) / kDegBound;
+        for (int k = 0; k < nseg; k++)
+            block4[at + k] = make_int4(d, (int)r, loc + k * kDegBound,
+                                       min(kDegBound, d - k * kDegBound));
+        return;
+    }
+    int w, rpb;
+    slice_rule(d, w, rpb);
+    if (((int)r - run_start[r]) % rpb != 0) return;
+    int n = 1;
+    while (n < rpb && r + n < rows && (int)deg[r + n] == d) n++;
+    block4[at] = make_int4(d, (int)r, loc, (w << 16) + n);
+}
+
+struct DevBuf {  // frees on scope exit
+    void *p = nullptr;
+    ~DevBuf() { if (p) (void)hipFree(p); }
+    int alloc(size_t bytes)
+    {
+        if (hipMalloc(&p, bytes ? bytes : 4) != hipSuccess) {
+            p = nullptr;
+            (void)hipGetLastError();
+            set_error("device allocation of %zu bytes failed", bytes);
+            return ACCEL_ERR_ALLOC;
+        }
+        return ACCEL_OK;
+    }
+    template <class T> T *as() { return static_cast<T *>(p); }
+    void *release() { void *q = p; p = nullptr; return q; }
+};
+
+inline unsigned grid_for(int64_t n) { return (unsigned)((n + kThreads - 1) / kThreads); }
+
+}  // namespace
+
+// Builds row_block[rows+1] and block4 from degrees given in partition order.
+// Outputs are freshly allocated device arrays (caller frees).  *n_blocks on host.
+static int partition_device(const uint32_t *deg, const int32_t *s_indptr, int64_t rows,
+                            int32_t **row_block_out, int32_t **block4_out, int64_t *n_blocks,
+                            hipStream_t s)
+{
+    DevBuf head, cnt, sums, rb, b4;
+    int rc;
+    if ((rc = head.alloc(sizeof(int) * (size_t)rows))) return rc;
+    if ((rc = cnt.alloc(sizeof(int) * (size_t)rows))) return rc;
+    if ((rc = sums.alloc(sizeof(int) * (size_t)(rows / kTile + 4)))) return rc;
+    if ((rc = rb.alloc(sizeof(int) * (size_t)(rows + 1)))) return rc;
+    run_head_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(deg, rows, head.as<int>());
+    if ((rc = device_scan<MaxOp, true>(head.as<int>(), rows, head.as<int>(), nullptr,
+                                       sums.as<int>(), s)))
+        return rc;
+    block_count_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(deg, head.as<int>(), rows,
+                                                                      cnt.as<int>());
+    if ((rc = device_scan<SumOp, false>(cnt.as<int>(), rows, rb.as<int>(), rb.as<int>() + rows,
+                                        sums.as<int>(), s)))
+        return rc;
+    int nb = 0;
+    ACCEL_HIP(hipMemcpyAsync(&nb, rb.as<int>() + rows, sizeof(int), hipMemcpyDeviceToHost, s));
+    ACCEL_HIP(hipStreamSynchronize(s));
+    if ((rc = b4.alloc(sizeof(int4) * (size_t)nb))) return rc;
+    emit_block4_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(
+        deg, s_indptr, head.as<int>(), rb.as<int>(), rows, b4.as<int4>());
+    ACCEL_HIP(hipGetLastError());
+    ACCEL_HIP(hipStreamSynchronize(s));
+    *n_blocks = nb;
+    *row_block_out = static_cast<int32_t *>(rb.release());
+    *block4_out = static_cast<int32_t *>(b4.release());
+    return ACCEL_OK;
+}
+
+// Partition a row order as given (no sort): the GPU counterpart of running
+// block_level_partition.py on one *.new_indptr file.
+int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
+                          int32_t **block4_dev, int64_t *n_blocks)
+{
+    hipStream_t s = nullptr;
+    DevBuf deg, st;
+    int rc;
+    if ((rc = deg.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
+    if ((rc = st.alloc(sizeof(Stats)))) return rc;
+    ACCEL_HIP(hipMemsetAsync(st.p, 0, sizeof(Stats), s));
+    degree_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(indptr_dev, rows, nnz,
+                                                                 deg.as<uint32_t>(), st.as<Stats>());
+    Stats hs;
+    ACCEL_HIP(hipMemcpyAsync(&hs, st.p, sizeof(Stats), hipMemcpyDeviceToHost, s));
+    ACCEL_HIP(hipStreamSynchronize(s));
+    if (hs.bad_indptr) {
+        set_error("indptr must start at 0, be non-decreasing and end at nnz");
+        return ACCEL_ERR_CSR;
+    }
+    int32_t *rb = nullptr;
+    rc = partition_device(deg.as<uint32_t>(), indptr_dev, rows, &rb, block4_dev, n_blocks, s);
+    if (rb) (void)hipFree(rb);
+    return rc;
+}
+
+int preprocess_device(accel_handle *h)
+{
+    const auto t0 = std::chrono::steady_clock::now();
+    hipStream_t s = nullptr;
+    const int64_t rows = h->rows, nnz = h->nnz;
+    int rc;
+
+    h->ready = false;
+    h->n_blocks = h->n_long_blocks = h->n_long_rows = h->n_zero_rows = 0;
+    h->max_degree = 0;
+    if (rows == 0) {
+        h->identity_perm = true;
+        h->ready = true;
+        return ACCEL_OK;
+    }
+
+    DevBuf deg, st;
+    if ((rc = deg.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
+    if ((rc = st.alloc(sizeof(Stats)))) return rc;
+    ACCEL_HIP(hipMemsetAsync(st.p, 0, sizeof(Stats), s));
+    degree_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(h->indptr, rows, nnz,
+                                                                 deg.as<uint32_t>(), st.as<Stats>());
+    Stats hs;
+    ACCEL_HIP(hipMemcpyAsync(&hs, st.p, sizeof(Stats), hipMemcpyDeviceToHost, s));
+    ACCEL_HIP(hipStreamSynchronize(s));
+    if (hs.bad_indptr) {   // checked before idx is touched: nnz is trusted from here on
+        set_error("indptr must start at 0, be non-decreasing and end at nnz");
+        return ACCEL_ERR_CSR;
+    }
+    if (nnz > 0) {
+        const unsigned g = (unsigned)std::min<int64_t>((nnz + kThreads - 1) / kThreads, 65536);
+        index_check_kernel<<<dim3(g), dim3(kThreads), 0, s>>>(h->idx, nnz, h->cols, st.as<Stats>());
+        ACCEL_HIP(hipMemcpyAsync(&hs, st.p, sizeof(Stats), hipMemcpyDeviceToHost, s));
+        ACCEL_HIP(hipStreamSynchronize(s));
+        if (hs.bad_index) {
+            set_error("a column index lies outside [0, cols)");
+            return ACCEL_ERR_CSR;
+        }
+    }
+    h->max_degree = hs.max_degree;
+    h->n_zero_rows = hs.n_zero_rows;
+    h->n_long_rows = hs.n_long_rows;
+    h->n_long_blocks = hs.n_long_blocks;
+    h->identity_perm = !hs.unsorted;
+
+    // ---- degree sort ------------------------------------------------------
+    DevBuf keys_b, vals_a, vals_b, hist, sums;
+    uint32_t *sdeg = deg.as<uint32_t>();
+    uint32_t *perm = nullptr;
+    if (!h->identity_perm) {
+        const int64_t tiles = (rows + kTile - 1) / kTile;
+        if ((rc = keys_b.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
+        if ((rc = vals_a.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
+        if ((rc = vals_b.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
+        if ((rc = hist.alloc(sizeof(int) * (size_t)(256 * tiles)))) return rc;
+        if ((rc = sums.alloc(sizeof(int) * (size_t)(256 * tiles / kTile + 4)))) return rc;
+        int bits = 0;
+        while (bits < 32 && (hs.max_degree >> bits) != 0) bits++;
+        uint32_t *kin = deg.as<uint32_t>(), *kout = keys_b.as<uint32_t>();
+        uint32_t *vin = nullptr, *vout = vals_a.as<uint32_t>();
+        for (int shift = 0; shift < bits; shift += 8) {
+            radix_hist<<<dim3((unsigned)tiles), dim3(kThreads), 0, s>>>(kin, rows, shift,
+                                                                       hist.as<int>(), tiles);
+            if ((rc = device_scan<SumOp, false>(hist.as<int>(), 256 * tiles, hist.as<int>(),
+                                                nullptr, sums.as<int>(), s)))
+                return rc;
+            radix_scatter<<<dim3((unsigned)tiles), dim3(kThreads), 0, s>>>(
+                kin, vin, kout, vout, rows, shift, hist.as<int>(), tiles);
+            std::swap(kin, kout);
+            vin = vout;
+            vout = (vout == vals_a.as<uint32_t>()) ? vals_b.as<uint32_t>() : vals_a.as<uint32_t>();
+        }
+        ACCEL_HIP(hipGetLastError());
+        sdeg = kin;
+        perm = vin;   // non-null: unsorted input has max_degree >= 1, so at least one pass ran
+    }
+
+    // ---- sorted indptr ------------------------------------------------------
+    DevBuf sip, ssums;
+    if ((rc = sip.alloc(sizeof(int32_t) * (size_t)(rows + 1)))) return rc;
+    if ((rc = ssums.alloc(sizeof(int) * (size_t)(rows / kTile + 4)))) return rc;
+    if ((rc = device_scan<SumOp, false>(reinterpret_cast<const int *>(sdeg), rows, sip.as<int>(),
+                                        sip.as<int>() + rows, ssums.as<int>(), s)))
+        return rc;
+
+    // ---- permuted CSR -------------------------------------------------------
+    DevBuf sidx, sval, permbuf;
+    if (!h->identity_perm) {
+        if ((rc = sidx.alloc(sizeof(int32_t) * (size_t)nnz))) return rc;
+        if ((rc = sval.alloc(sizeof(float) * (size_t)nnz))) return rc;
+        if (nnz > 0)
+            permute_csr_kernel<<<dim3(grid_for(nnz)), dim3(kThreads), 0, s>>>(
+                h->indptr, h->idx, h->val, reinterpret_cast<const int32_t *>(perm), sip.as<int32_t>(),
+                rows, nnz, sidx.as<int32_t>(), sval.as<float>());
+        if ((rc = permbuf.alloc(sizeof(int32_t) * (size_t)rows))) return rc;
+        ACCEL_HIP(hipMemcpyAsync(permbuf.p, perm, sizeof(int32_t) * (size_t)rows,
+                                 hipMemcpyDeviceToDevice, s));
+        ACCEL_HIP(hipGetLastError());
+    }
+
+    // ---- partition ----------------------------------------------------------
+    int32_t *rb = nullptr, *b4 = nullptr;
+    int64_t nb = 0;
+    if ((rc = partition_device(sdeg, sip.as<int32_t>(), rows, &rb, &b4, &nb, s))) return rc;
+    ACCEL_HIP(hipStreamSynchronize(s));
+
+    h->row_block = rb;
+    h->block4 = b4;
+    h->n_blocks = nb;
+    h->s_indptr = static_cast<int32_t *>(sip.release());
+    if (h->identity_perm) {
+        h->perm = nullptr;
+        h->s_idx = h->idx;
+        h->s_val = h->val;
+        h->owns_sorted = false;
+    } else {
+        h->perm = static_cast<int32_t *>(permbuf.release());
+        h->s_idx = static_cast<int32_t *>(sidx.release());
+        h->s_val = static_cast<float *>(sval.release());
+        h->owns_sorted = true;
+    }
+    h->ready = true;
+    h->preprocess_ms =
+        std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    return ACCEL_OK;
+}
+
+}  // namespace accel

@@ -1,0 +1,331 @@
+// The SpMM gather kernel for gfx950 (wave64) and its two helpers.
+//
+// Work decomposition.  The unit of work is one block4 entry (upstream's
+// spmm_accel.cu:18-28 gives one CUDA thread block of 12 32-lane warps to each
+// entry); here one 64-lane wavefront takes one entry and a 256-thread workgroup
+// takes four consecutive entries.  An entry is either up to 12 whole rows of one
+// degree (<= 384 non-zeros in total) or one <= 384-non-zero segment of a row with
+// more than 384 non-zeros.
+//
+// Inside the wavefront the lanes form G = 64 / L groups of L lanes; a group owns
+// L * VEC consecutive columns of X/Y (VEC = 4 floats = one 16-byte load per lane
+// when N allows), so one vector-memory instruction gathers G different rows of X.
+// This replaces upstream's "combined warp" of ceil32(N) lanes that walks one
+// non-zero at a time with 4-byte loads (spmm_accel.cu:37-48,56-78).  G groups are
+// split over the entry's rows as gp groups per row (gp a power of two chosen per
+// entry to minimise the step count); the gp partial sums of a row are combined by
+// a cross-lane butterfly, so short rows need no atomics (upstream: atomicAdd for
+// every row that spans more than one warp, spmm_accel.cu:82-99).
+//
+// The (column index, value) pairs of the entry are first staged in LDS with
+// coalesced loads, one pair per lane; each group then reads its pairs back with
+// broadcast LDS reads.  Segments of long rows write their partial sums to a
+// scratch buffer and a second small kernel adds them up in a fixed order, so the
+// result is run-to-run deterministic.  Rows of degree 0 are zero-filled by extra
+// workgroups of the same launch: Y = A X holds after every run with no memset.
+#include "internal.h"
+
+namespace accel {
+namespace {
+
+constexpr int kWaves = 4;                 // wavefronts (= block4 entries) per workgroup
+constexpr int kWgThreads = 64 * kWaves;
+constexpr int kZeroFloats = 16384;        // floats zero-filled per extra workgroup
+
+template <int VEC>
+__device__ __forceinline__ void load_vec(const float *__restrict__ p, float (&v)[VEC])
+{
+    if constexpr (VEC == 4) {
+        const float4 t = *reinterpret_cast<const float4 *>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else if constexpr (VEC == 2) {
+        const float2 t = *reinterpret_cast<const float2 *>(p);
+        v[0] = t.x; v[1] = t.y;
+    } else {
+        v[0] = *p;
+    }
+}
+
+template <int VEC>
+__device__ __forceinline__ void store_vec(float *__restrict__ p, const float (&v)[VEC])
+{
+    if constexpr (VEC == 4) {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    } else if constexpr (VEC == 2) {
+        *reinterpret_cast<float2 *>(p) = make_float2(v[0], v[1]);
+    } else {
+        *p = v[0];
+    }
+}
+
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+template <int L, int VEC>
+__global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
+    const int4 *__restrict__ block4, int n_blocks, int n_short_blocks,
+    const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
+    const int32_t *__restrict__ perm, const float *__restrict__ X, float *__restrict__ Y,
+    float *__restrict__ partial, int N, int n_zero_rows, int n_entry_groups)
+{
+    constexpr int G = 64 / L;        // lane groups per wavefront
+    constexpr int CW = L * VEC;      // columns covered per pass
+    __shared__ int2 stage[kWaves][kDegBound];
+
+    if ((int)blockIdx.x >= n_entry_groups) {
+        // zero-degree rows: they are the first n_zero_rows rows of the sorted order
+        const int64_t first = (int64_t)(blockIdx.x - n_entry_groups) * kZeroFloats;
+        const int64_t total = (int64_t)n_zero_rows * N;
+        for (int64_t i = first + threadIdx.x; i < first + kZeroFloats && i < total; i += kWgThreads) {
+            const int64_t r = i / N;
+            const int64_t c = i - r * N;
+            const int64_t out_row = perm ? perm[r] : r;
+            Y[out_row * N + c] = 0.0f;
+        }
+        return;
+    }
+
+    const int lane = threadIdx.x & 63;
+    const int wv = uniform(threadIdx.x >> 6);
+    int e = (int)blockIdx.x * kWaves + wv;
+    if (e >= n_blocks) return;
+    e = n_blocks - 1 - e;            // heaviest entries (long-row segments) are scheduled first
+
+    const int4 b = block4[e];
+    const int deg = uniform(b.x), row0 = uniform(b.y), loc = uniform(b.z), info = uniform(b.w);
+    const bool is_long = deg > kDegBound;
+    const int n_rows = is_long ? 1 : (info & 0xFFFF);   // spmm_accel.cu:26
+    const int d = is_long ? info : deg;                 // spmm_accel.cu:28: non-zeros per row here
+    const int total_nz = n_rows * d;
+
+    // stage the entry's (column, value) pairs: all loads are issued before the first LDS write
+    int2 *st = stage[wv];
+    {
+        constexpr int kRounds = kDegBound / 64;
+        int ci[kRounds];
+        float cv[kRounds];
+#pragma unroll
+        for (int j = 0; j < kRounds; j++) {
+            const int i = lane + 64 * j;
+            if (i < total_nz) {
+                ci[j] = s_idx[loc + i];
+                cv[j] = s_val[loc + i];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kRounds; j++) {
+            const int i = lane + 64 * j;
+            if (i < total_nz) st[i] = make_int2(ci[j], __float_as_int(cv[j]));
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+
+    // groups per row: power of two that minimises ceil(n_rows / (G/gp)) * ceil(d / gp)
+    int lg = 0;
+    if constexpr (G > 1) {
+        int best = 0x7fffffff;
+#pragma unroll
+        for (int q = 0; (1 << q) <= G; q++) {
+            const int rows_at_once = G >> q;
+            const int steps = ((n_rows + rows_at_once - 1) / rows_at_once) * ((d + (1 << q) - 1) >> q);
+            if (steps < best) { best = steps; lg = q; }
+        }
+    }
+    const int gp = 1 << lg;
+    const int rows_at_once = G >> lg;
+    const int g = lane / L, sub = lane % L;
+    const int k = g & (gp - 1);          // which of the row's gp groups this is
+    const int rloc = g >> lg;            // which of the rows in flight
+
+    for (int c0 = 0; c0 < N; c0 += CW) {
+        const int col = c0 + sub * VEC;
+        const bool col_ok = col < N;
+        for (int r_it = 0; r_it < n_rows; r_it += rows_at_once) {
+            const int r = r_it + rloc;
+            const bool live = col_ok && r < n_rows;
+            float acc[VEC];
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[v] = 0.0f;
+            if (live) {
+                const int2 *row_st = st + r * d;
+                const float *xcol = X + col;
+                int o = k;
+                for (; o + 3 * gp < d; o += 4 * gp) {
+                    int2 p[4];
+                    float x[4][VEC];
+#pragma unroll
+                    for (int u = 0; u < 4; u++) p[u] = row_st[o + u * gp];
+#pragma unroll
+                    for (int u = 0; u < 4; u++) load_vec<VEC>(xcol + (int64_t)p[u].x * N, x[u]);
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const float a = __int_as_float(p[u].y);
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[u][v], acc[v]);
+                    }
+                }
+                for (; o < d; o += gp) {
+                    const int2 p = row_st[o];
+                    float x[VEC];
+                    load_vec<VEC>(xcol + (int64_t)p.x * N, x);
+                    const float a = __int_as_float(p.y);
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[v], acc[v]);
+                }
+            }
+            // add the gp partial sums of each row (all lanes take part)
+            for (int m = L; m < (L << lg); m <<= 1) {
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[v] += __shfl_xor(acc[v], m);
+            }
+            if (live && k == 0) {
+                if (is_long) {
+                    store_vec<VEC>(partial + (int64_t)(e - n_short_blocks) * N + col, acc);
+                } else {
+                    const int64_t out_row = perm ? perm[row0 + r] : row0 + r;
+                    store_vec<VEC>(Y + out_row * N + col, acc);
+                }
+            }
+        }
+    }
+}
+
+// Adds the segment partials of each long row in segment order and writes the row.
+__global__ __launch_bounds__(kWgThreads) void long_row_reduce_kernel(
+    const float *__restrict__ partial, const int32_t *__restrict__ s_indptr,
+    const int32_t *__restrict__ row_block, const int32_t *__restrict__ perm, int64_t first_long_row,
+    int n_short_blocks, float *__restrict__ Y, int N)
+{
+    __shared__ float red[kWgThreads];
+    const int64_t r = first_long_row + blockIdx.x;
+    const int d = s_indptr[r + 1] - s_indptr[r];
+    const int nseg = (d + kDegBound - 1) / kDegBound;
+    const float *src = partial + (int64_t)(row_block[r] - n_short_blocks) * N;
+    const int64_t out_row = perm ? perm[r] : r;
+    int cw = 1;                                   // columns per pass: power of two <= 256
+    while (cw < N && cw < kWgThreads) cw <<= 1;
+    const int sg = kWgThreads / cw;               // segment groups
+    const int c_in = threadIdx.x % cw, my_sg = threadIdx.x / cw;
+    for (int c0 = 0; c0 < N; c0 += cw) {
+        const int c = c0 + c_in;
+        float acc = 0.0f;
+        if (c < N)
+            for (int sgm = my_sg; sgm < nseg; sgm += sg) acc += src[(int64_t)sgm * N + c];
+        red[threadIdx.x] = acc;
+        __syncthreads();
+        if (my_sg == 0 && c < N) {
+            float t = acc;
+            for (int q = 1; q < sg; q++) t += red[q * cw + c_in];
+            Y[out_row * N + c] = t;
+        }
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t *dst, uint32_t v, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+        dst[i] = v;
+}
+
+template <int VEC>
+int launch_for_vec(int L, dim3 grid, hipStream_t s, const int4 *block4, int n_blocks, int n_short,
+                   const int32_t *s_idx, const float *s_val, const int32_t *perm, const float *X,
+                   float *Y, float *partial, int N, int n_zero_rows, int n_entry_groups)
+{
+#define ACCEL_LAUNCH(LL)                                                                      \
+    case LL:                                                                                  \
+        spmm_gather_kernel<LL, VEC><<<grid, dim3(kWgThreads), 0, s>>>(                        \
+            block4, n_blocks, n_short, s_idx, s_val, perm, X, Y, partial, N, n_zero_rows,     \
+            n_entry_groups);                                                                  \
+        break;
+    switch (L) {
+        ACCEL_LAUNCH(1)
+        ACCEL_LAUNCH(2)
+        ACCEL_LAUNCH(4)
+        ACCEL_LAUNCH(8)
+        ACCEL_LAUNCH(16)
+        ACCEL_LAUNCH(32)
+        ACCEL_LAUNCH(64)
+    default:
+        set_error("internal: unsupported group width %d", L);
+        return ACCEL_ERR_ARG;
+    }
+#undef ACCEL_LAUNCH
+    return ACCEL_OK;
+}
+
+}  // namespace
+
+int fill_u32(void *dst, uint32_t v, size_t n, hipStream_t s)
+{
+    if (n == 0) return ACCEL_OK;
+    const unsigned g = (unsigned)std::min<size_t>((n + 255) / 256, 4096);
+    fill_u32_kernel<<<dim3(g), dim3(256), 0, s>>>(static_cast<uint32_t *>(dst), v, n);
+    ACCEL_HIP(hipGetLastError());
+    return ACCEL_OK;
+}
+
+int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
+                hipEvent_t after_main)
+{
+    if (h->rows == 0) return ACCEL_OK;
+    // widest vector the row stride and the base pointers allow
+    const uintptr_t align = reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Y);
+    int vec = 1;
+    if (N % 4 == 0 && align % 16 == 0) vec = 4;
+    else if (N % 2 == 0 && align % 8 == 0) vec = 2;
+    int L = 1;
+    while (L * vec < N && L < 64) L <<= 1;
+
+    const int64_t n_short = h->n_blocks - h->n_long_blocks;
+    if (h->n_long_blocks > 0) {
+        const size_t need = (size_t)h->n_long_blocks * (size_t)N;
+        if (h->partial_floats < need) {
+            if (h->partial) (void)hipFree(h->partial);
+            h->partial = nullptr;
+            h->partial_floats = 0;
+            if (hipMalloc(reinterpret_cast<void **>(&h->partial), need * sizeof(float)) != hipSuccess) {
+                (void)hipGetLastError();
+                set_error("device allocation of %zu bytes for long-row partial sums failed",
+                          need * sizeof(float));
+                return ACCEL_ERR_ALLOC;
+            }
+            h->partial_floats = need;
+        }
+    }
+    const int64_t entry_groups = (h->n_blocks + kWaves - 1) / kWaves;
+    const int64_t zero_groups = (h->n_zero_rows * (int64_t)N + kZeroFloats - 1) / kZeroFloats;
+    const int64_t groups = entry_groups + zero_groups;
+    if (groups > 0x7fffffffLL) {
+        set_error("launch of %lld workgroups exceeds the grid limit", (long long)groups);
+        return ACCEL_ERR_ARG;
+    }
+    int rc = ACCEL_OK;
+    if (groups > 0) {
+        const dim3 grid((unsigned)groups);
+        const int4 *b4 = reinterpret_cast<const int4 *>(h->block4);
+        if (vec == 4)
+            rc = launch_for_vec<4>(L, grid, stream, b4, (int)h->n_blocks, (int)n_short, h->s_idx,
+                                   h->s_val, h->perm, X, Y, h->partial, N, (int)h->n_zero_rows,
+                                   (int)entry_groups);
+        else if (vec == 2)
+            rc = launch_for_vec<2>(L, grid, stream, b4, (int)h->n_blocks, (int)n_short, h->s_idx,
+                                   h->s_val, h->perm, X, Y, h->partial, N, (int)h->n_zero_rows,
+                                   (int)entry_groups);
+        else
+            rc = launch_for_vec<1>(L, grid, stream, b4, (int)h->n_blocks, (int)n_short, h->s_idx,
+                                   h->s_val, h->perm, X, Y, h->partial, N, (int)h->n_zero_rows,
+                                   (int)entry_groups);
+        if (rc) return rc;
+    }
+    if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));
+    if (h->n_long_rows > 0) {
+        long_row_reduce_kernel<<<dim3((unsigned)h->n_long_rows), dim3(kWgThreads), 0, stream>>>(
+            h->partial, h->s_indptr, h->row_block, h->perm, h->rows - h->n_long_rows, (int)n_short,
+            Y, N);
+    }
+    ACCEL_HIP(hipGetLastError());
+    return ACCEL_OK;
+}
+
+}  // namespace accel

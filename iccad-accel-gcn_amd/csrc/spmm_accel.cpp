@@ -1,0 +1,56 @@
+// SPMM_ACCEL over the C ABI (see include/spmm_accel.h).
+#include "spmm_accel.h"
+
+#include <vector>
+
+#include "accel_gcn.h"
+
+SPMM_ACCEL::~SPMM_ACCEL()
+{
+    if (h) accel_destroy(h);
+}
+
+bool SPMM_ACCEL::preprocess()
+{
+    if (h) return true;
+    err.clear();
+    int rc = accel_create(ptr, idx, val, num_v, num_v, num_e, ACCEL_PTR_DEVICE, &h);
+    if (!rc) rc = accel_preprocess(h);
+    accel_info info{};
+    if (!rc) rc = accel_get_info(h, &info);
+    if (!rc) {
+        n_blocks = info.n_blocks;
+        // a .block4 file written for this graph must describe the same partition
+        const std::string path = meta_dir + _graph + ".block4";
+        int64_t n = 0;
+        if (accel_file_count(path.c_str(), &n) == ACCEL_OK) {
+            std::vector<int32_t> file((size_t)n);
+            rc = accel_file_read(path.c_str(), file.data(), n);
+            if (!rc && n % 4 != 0) rc = ACCEL_ERR_META;
+            if (!rc) rc = accel_check_block4(h, file.data(), n / 4);
+        }
+    }
+    if (rc) {
+        err = accel_last_error();
+        if (h) accel_destroy(h);
+        h = nullptr;
+        return false;
+    }
+    // launch geometry, for callers that print it: 4 entries per 256-thread workgroup
+    grid.x = (unsigned)((n_blocks + 3) / 4);
+    block.x = 256;
+    return true;
+}
+
+void SPMM_ACCEL::run(int dim)
+{
+    if (!h) return;
+    if (accel_run(h, vin, vout, dim, nullptr) != ACCEL_OK) err = accel_last_error();
+}
+
+double SPMM_ACCEL::do_test(bool timing, int dim)
+{
+    if (!preprocess()) return -1.0;
+    const double t = timing_body(timing, dim);
+    return err.empty() ? t : -1.0;
+}

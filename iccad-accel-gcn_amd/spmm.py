@@ -1,0 +1,194 @@
+"""Host-side mirror of the operator interface for Python callers.
+
+``SpmmAccel`` follows upstream's SPMM_ACCEL (spmm_accel.h:4-20) through
+SPMM_BASE (spmm_base.h:6-65): construct on (graph, ptr, idx, val, vin, vout,
+num_v, num_e, dim), then ``do_test(timing, dim)`` preprocesses and runs, and
+``run(dim)`` is one asynchronous launch.  ``AccelSpMM`` is the numpy-friendly
+wrapper used by tests and the benchmark: init / preprocess / run.
+
+Everything computes through the C ABI of libaccelgcn.so on the GPU.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import time
+from pathlib import Path
+
+import numpy as np
+
+from . import _lib
+from ._lib import AccelError, DeviceBuffer, Info, check, lib, ptr
+
+
+class AccelSpMM:
+    """Y = A @ X for a CSR matrix A (int32 indices, fp32 values) on the GPU.
+
+    init: ``AccelSpMM(indptr, indices, values, n_cols)`` uploads the CSR (host
+    numpy arrays) or borrows it (``device=True``: objects with ``data_ptr()`` or
+    raw addresses, plus explicit ``n_rows``/``nnz``).
+    preprocess: ``preprocess()`` degree-sorts and partitions on the GPU.
+    run: ``run(X, Y, N)`` on device buffers, or ``matmul(X)`` numpy -> numpy.
+    """
+
+    def __init__(self, indptr, indices, values, n_cols, *, device=False, n_rows=None, nnz=None):
+        self._h = C.c_void_p()
+        self._keep = None
+        if device:
+            if n_rows is None or nnz is None:
+                raise ValueError("device=True needs n_rows and nnz")
+            self.n_rows, self.nnz = int(n_rows), int(nnz)
+            self._keep = (indptr, indices, values)
+            args = (ptr(indptr), ptr(indices), ptr(values))
+            flags = _lib.PTR_DEVICE
+        else:
+            ip = _lib.as_i32(indptr)
+            ix = _lib.as_i32(indices)
+            v = _lib.as_f32(values)
+            if ip.ndim != 1 or ip.size < 1:
+                raise AccelError(_lib.ERR_ARG, "indptr must be a 1-D array with at least one entry")
+            if ix.size != v.size:
+                raise AccelError(_lib.ERR_ARG, "indices and values differ in length")
+            self.n_rows, self.nnz = ip.size - 1, ix.size
+            self._keep = (ip, ix, v)
+            args = (ptr(ip), ptr(ix), ptr(v))
+            flags = _lib.PTR_HOST
+        self.n_cols = int(n_cols)
+        check(lib().accel_create(*args, self.n_rows, self.n_cols, self.nnz, flags, C.byref(self._h)))
+        if not device:
+            self._keep = None       # uploaded: host copies are no longer needed
+        self._info = None
+
+    # -- preprocess ---------------------------------------------------------
+    def preprocess(self) -> "AccelSpMM":
+        check(lib().accel_preprocess(self._h))
+        info = Info()
+        check(lib().accel_get_info(self._h, C.byref(info)))
+        self._info = info
+        return self
+
+    @property
+    def info(self) -> Info:
+        if self._info is None:
+            raise AccelError(_lib.ERR_STATE, "call preprocess() first")
+        return self._info
+
+    def block4(self) -> np.ndarray:
+        out = np.empty((self.info.n_blocks, 4), dtype=np.int32)
+        check(lib().accel_get_block4(self._h, ptr(out, C.c_int32), out.shape[0]))
+        return out
+
+    def perm(self) -> np.ndarray:
+        self.info
+        out = np.empty(self.n_rows, dtype=np.int32)
+        check(lib().accel_get_perm(self._h, ptr(out, C.c_int32), out.size))
+        return out
+
+    def sorted_csr(self):
+        self.info
+        ip = np.empty(self.n_rows + 1, dtype=np.int32)
+        ix = np.empty(self.nnz, dtype=np.int32)
+        v = np.empty(self.nnz, dtype=np.float32)
+        check(lib().accel_get_sorted_csr(self._h, ptr(ip, C.c_int32), ptr(ix, C.c_int32), ptr(v, C.c_float)))
+        return ip, ix, v
+
+    def check_block4(self, block4) -> None:
+        b = _lib.as_i32(block4).reshape(-1)
+        if b.size % 4:
+            raise AccelError(_lib.ERR_META, "metadata length is not a multiple of 4")
+        check(lib().accel_check_block4(self._h, ptr(b, C.c_int32), b.size // 4))
+
+    # -- run ----------------------------------------------------------------
+    def run(self, X, Y, N: int, stream=None) -> None:
+        """One asynchronous launch; X, Y are device buffers."""
+        check(lib().accel_run(self._h, ptr(X), ptr(Y), int(N), ptr(stream)))
+
+    def synchronize(self, stream=None) -> None:
+        check(lib().accel_stream_sync(ptr(stream)))
+
+    def matmul(self, X: np.ndarray) -> np.ndarray:
+        X = _lib.as_f32(X)
+        if X.ndim != 2 or X.shape[0] != self.n_cols:
+            raise AccelError(_lib.ERR_ARG, f"X must be [{self.n_cols}, N]")
+        N = X.shape[1]
+        dX = DeviceBuffer.from_numpy(X)
+        dY = DeviceBuffer(max(self.n_rows * N * 4, 4))
+        dY.fill_u32(0x7FC00000)          # NaN: any row the operator fails to write shows up
+        try:
+            self.run(dX, dY, N)
+            self.synchronize()
+            return dY.to_numpy(np.float32, (self.n_rows, N))
+        finally:
+            dX.close()
+            dY.close()
+
+    def time(self, X, Y, N: int, warmup: int = 4, iters: int = 20, stream=None):
+        """HIP-event timings in ms: (total per run, gather kernel only)."""
+        tot = np.zeros(iters, dtype=np.float32)
+        main = np.zeros(iters, dtype=np.float32)
+        check(lib().accel_time(self._h, ptr(X), ptr(Y), int(N), warmup, iters,
+                               ptr(tot, C.c_float), ptr(main, C.c_float), ptr(stream)))
+        return tot, main
+
+    def close(self) -> None:
+        if self._h:
+            lib().accel_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class SpmmAccel:
+    """Python mirror of SPMM_ACCEL (spmm_accel.h:4-20, spmm_base.h:9-23).
+
+    All array arguments are device pointers (DeviceBuffer, objects with
+    ``data_ptr()``, or addresses), exactly as upstream's main.cu:131 passes
+    managed-memory pointers.  ``do_test`` returns mean seconds per launch over
+    the 4-warm-up / 4-timed host-clock protocol (spmm_base.h:44-60), 0.0 when
+    ``timing`` is false.
+    """
+
+    def __init__(self, graph, ptr_, idx, val, vin, vout, num_v, num_e, dim, meta_dir="../block_level_meta/"):
+        self._graph = graph
+        self.vin, self.vout = vin, vout
+        self.num_v, self.num_e, self.dim = int(num_v), int(num_e), int(dim)
+        self.meta_dir = Path(meta_dir)
+        self._op = AccelSpMM(ptr_, idx, val, self.num_v, device=True, n_rows=self.num_v, nnz=self.num_e)
+        self._ready = False
+
+    def _preprocess(self):
+        if self._ready:
+            return
+        self._op.preprocess()
+        meta = self.meta_dir / f"{self._graph}.block4"
+        if meta.exists():      # a stale file must not pass silently (spmm_accel.cu:122 trusts it blindly)
+            self._op.check_block4(np.fromfile(meta, dtype="<i4"))
+        self._ready = True
+
+    def run(self, dim):
+        self._op.run(self.vin, self.vout, dim)
+
+    def do_test(self, timing: bool, dim: int) -> float:
+        self._preprocess()
+        if not timing:
+            self.run(dim)
+            self._op.synchronize()
+            return 0.0
+        times = 4
+        for _ in range(times):
+            self.run(dim)
+        self._op.synchronize()
+        total = 0.0
+        for _ in range(times):
+            t0 = time.perf_counter()
+            self.run(dim)
+            self._op.synchronize()
+            total += time.perf_counter() - t0
+        return total / times
+
+    @property
+    def op(self) -> AccelSpMM:
+        return self._op

@@ -1,0 +1,149 @@
+/*
+ * accel_gcn.h - C ABI of the MI355X (gfx950) build of Accel-GCN's SpMM hot path.
+ *
+ * The path: Y = A * X, A a CSR adjacency (int32 indices, fp32 values), X and Y
+ * dense row-major fp32 with N columns; rows are degree-sorted and cut into
+ * blocks of at most 384 non-zeros described by int32 quadruples (the ".block4"
+ * metadata).  Every entry point below names the upstream interface it replaces
+ * (paths relative to the upstream tree).
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every function returns an accel_status
+ *     (0 = ok, negative = error) and accel_last_error() describes the last
+ *     failure on the calling thread;
+ *   - a handle is not thread-safe; distinct handles are independent;
+ *   - "device pointer" = anything the GPU can dereference (hipMalloc,
+ *     hipMallocManaged, as upstream's data.h:15 uses);
+ *   - nothing here falls back to the CPU: the *_host functions are explicit
+ *     host utilities, every other call needs a GPU and fails with
+ *     ACCEL_ERR_HIP without one.
+ */
+#ifndef ACCEL_GCN_H
+#define ACCEL_GCN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum accel_status {
+    ACCEL_OK = 0,
+    ACCEL_ERR_ARG = -1,    /* null pointer, non-positive size, N <= 0, ... */
+    ACCEL_ERR_CSR = -2,    /* indptr not monotone / not starting at 0 / not ending at nnz, column out of range */
+    ACCEL_ERR_ALLOC = -3,  /* host or device allocation failed */
+    ACCEL_ERR_HIP = -4,    /* HIP runtime error (includes "no GPU") */
+    ACCEL_ERR_META = -5,   /* supplied .block4 metadata does not describe this CSR */
+    ACCEL_ERR_STATE = -6,  /* call order violated (run before preprocess, ...) */
+    ACCEL_ERR_IO = -7      /* file missing / truncated */
+} accel_status;
+
+/* accel_create flags */
+#define ACCEL_PTR_HOST 0   /* indptr/idx/val are host arrays: copied to the GPU */
+#define ACCEL_PTR_DEVICE 1 /* device pointers: borrowed, must outlive the handle */
+
+/* metadata ABI shared with upstream (spmm_accel.cu:11-12, block_level_partition.py:7-8) */
+#define ACCEL_DEG_BOUND 384
+#define ACCEL_SLICES_PER_BLOCK 12
+
+typedef struct accel_handle accel_handle;
+
+/* Message for the most recent error on this thread ("" if none). */
+const char *accel_last_error(void);
+/* Library version, major*10000 + minor*100 + patch. */
+int accel_version(void);
+
+/* ---- host utilities -------------------------------------------------------
+ * accel_partition_host: the walk of block_level_partition.py:48-103 with the
+ * tables of :7-21, on the host.  Writes up to cap quadruples
+ * (degree,row_begin,loc_begin,info) to block4_out (may be NULL with cap 0 to
+ * size the buffer) and the full count to *n_blocks.
+ * accel_degree_sort_host: perm_out[new_row] = old_row, ascending degree, ties
+ * by row id: the order upstream's *.new_indptr files are in
+ * (block_level_partition.py:31,38; tie-break defined by this library). */
+int accel_partition_host(const int32_t *indptr, int64_t rows, int32_t *block4_out, int64_t cap,
+                         int64_t *n_blocks);
+int accel_degree_sort_host(const int32_t *indptr, int64_t rows, int32_t *perm_out);
+
+/* The same partition computed by HIP kernels (scans + one emit kernel) for a
+ * host indptr in the row order given, i.e. what block_level_partition.py:38-106
+ * produces for one *.new_indptr file.  Bit-exact with accel_partition_host. */
+int accel_partition_gpu(const int32_t *indptr, int64_t rows, int32_t *block4_out, int64_t cap,
+                        int64_t *n_blocks);
+
+/* ---- raw-array files (data.h:7-34; block_level_partition.py:31-32,105-106) --
+ * Whole-file little-endian arrays of 4-byte elements.  accel_file_count
+ * returns the element count; accel_file_read fills a host buffer. */
+int accel_file_count(const char *path, int64_t *n_elems);
+int accel_file_read(const char *path, void *dst, int64_t n_elems);
+int accel_file_write(const char *path, const void *src, int64_t n_elems);
+
+/* ---- device memory plumbing (for callers without a HIP binding of their own;
+ * upstream uses cudaMallocManaged/cudaFree directly, main.cu:62-88,171-181) -- */
+int accel_device_count(int *n);
+int accel_dev_malloc(void **p, size_t bytes);
+int accel_dev_free(void *p);
+int accel_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes);
+int accel_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes);
+int accel_dev_fill_u32(void *dst_dev, uint32_t value, size_t n_words, void *stream);
+int accel_stream_sync(void *stream); /* NULL = default stream */
+
+/* ---- the operator ----------------------------------------------------------
+ * init: replaces SPMM_BASE's constructor (spmm_base.h:9-20) for the CSR part:
+ * stores (ACCEL_PTR_DEVICE) or uploads (ACCEL_PTR_HOST) the CSR.  The CSR may
+ * be in any row order. */
+int accel_create(const int32_t *indptr, const int32_t *idx, const float *val, int64_t rows,
+                 int64_t cols, int64_t nnz, int flags, accel_handle **out);
+
+/* preprocess: replaces the first half of SPMM_ACCEL::do_test (spmm_accel.cu:
+ * 122-132, which loads a .block4 file written by block_level_partition.py) and
+ * the offline degree sort behind upstream's *.new_* files.  On the GPU:
+ * validates the CSR, stable-sorts rows by degree (skipped when already
+ * sorted), gathers the permuted CSR, and builds the block4 metadata. */
+int accel_preprocess(accel_handle *h);
+
+/* Check externally produced metadata (a .block4 file) against what
+ * accel_preprocess built for this CSR; ACCEL_ERR_META if any int differs. */
+int accel_check_block4(accel_handle *h, const int32_t *block4_host, int64_t n_blocks);
+
+typedef struct accel_info {
+    int64_t rows, cols, nnz;
+    int64_t n_blocks;       /* block4 entries */
+    int64_t n_long_blocks;  /* entries that are segments of rows with degree > 384 */
+    int64_t n_long_rows;    /* rows with degree > 384 */
+    int64_t n_zero_rows;    /* rows with degree 0 */
+    int32_t max_degree;
+    int32_t already_sorted; /* 1: input rows were already in ascending degree order */
+    double preprocess_ms;   /* wall time of the last accel_preprocess */
+} accel_info;
+int accel_get_info(const accel_handle *h, accel_info *out);
+
+/* Copies to host: block4 (4*n_blocks int32), perm (rows int32), and the
+ * degree-sorted CSR (rows+1 / nnz / nnz); any pointer may be NULL to skip. */
+int accel_get_block4(const accel_handle *h, int32_t *out, int64_t cap_blocks);
+int accel_get_perm(const accel_handle *h, int32_t *out, int64_t cap_rows);
+int accel_get_sorted_csr(const accel_handle *h, int32_t *indptr, int32_t *idx, float *val);
+
+/* run: replaces SPMM_ACCEL::run (spmm_accel.cu:104-108).  Y = A X with beta = 0:
+ * every row of Y is written exactly once, rows of degree 0 receive zeros (the
+ * upstream kernel leaves them untouched and accumulates into the rest,
+ * spmm_accel.cu:84,97).  X has cols(A) rows, Y has rows(A) rows, both with
+ * leading dimension N (spmm_accel.cu:75,84 index row*feat_in+lane).  Rows of Y
+ * are in the caller's original row order.  Asynchronous on `stream` (a
+ * hipStream_t, NULL = default stream); X and Y are device pointers. */
+int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream);
+
+/* Timing protocol of SPMM_BASE::timing_body (spmm_base.h:34-63) with HIP
+ * events on `stream`: `warmup` untimed runs, then `iters` runs each bracketed
+ * by events.  ms_total[i] covers everything accel_run launches; ms_main[i]
+ * (optional) only the gather kernel.  Either array may be NULL. */
+int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup, int iters,
+               float *ms_total, float *ms_main, void *stream);
+
+int accel_destroy(accel_handle *h);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ACCEL_GCN_H */

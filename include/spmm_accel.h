@@ -1,0 +1,52 @@
+/*
+ * SPMM_ACCEL: the degree-sorted, block-partitioned SpMM operator behind the
+ * SPMM_BASE interface (upstream: spmm_accel.h:4-20, spmm_accel.cu:104-139).
+ *
+ * Construct it exactly as upstream's main.cu:131 does:
+ *     SPMM_ACCEL accel(graph, indptr, indices, val, vin, vout, v_num, e_num, dim_max);
+ * All six arrays are borrowed device-accessible pointers (hipMalloc or
+ * hipMallocManaged, as data.h:15 allocates them).
+ *
+ * do_test(timing, dim): preprocess + run, like spmm_accel.cu:110-139.  Upstream
+ * re-reads "../block_level_meta/<graph>.block4" on every call; here the degree
+ * sort and the metadata are built on the GPU once and cached in the object.  If
+ * that file exists it is compared with the GPU-built metadata and a mismatch is
+ * an error (do_test returns -1), so a stale file cannot silently mis-index.
+ * run(dim): one asynchronous launch; vout = A * vin with leading dimension dim.
+ *
+ * Differences from upstream that a caller can observe:
+ *   - vout is overwritten (beta = 0), zero-degree rows become 0; upstream
+ *     accumulates into vout and skips those rows (spmm_accel.cu:84,97);
+ *   - the CSR may be in any row order; vout rows follow the CSR given;
+ *   - any dim >= 1 works (upstream's lane mapping breaks for e.g. dim 130).
+ */
+#pragma once
+#include "spmm_base.h"
+
+struct accel_handle;
+
+class SPMM_ACCEL : public SPMM_BASE
+{
+public:
+    using SPMM_BASE::SPMM_BASE;
+    ~SPMM_ACCEL();
+
+    float *vout_ref = nullptr;   /* kept for source compatibility; unused */
+
+    double do_test(bool timing, int dim) override;
+    /* Directory searched for "<graph>.block4" (default: upstream's relative path). */
+    void set_meta_dir(const std::string &dir) { meta_dir = dir; }
+    /* Text of the last error ("" if none). */
+    const std::string &error() const { return err; }
+    /* Number of block4 entries after preprocessing. */
+    long long block_count() const { return n_blocks; }
+
+protected:
+    void run(int dim) override;
+
+    accel_handle *h = nullptr;
+    std::string meta_dir = "../block_level_meta/";
+    std::string err;
+    long long n_blocks = 0;
+    bool preprocess();
+};

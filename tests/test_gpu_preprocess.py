@@ -1,0 +1,168 @@
+"""GPU preprocessing (degree sort, permuted CSR, block4 partition) is bit-exact
+with the CPU oracle and with the reference's 16 golden .block4 files."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import block4_codec
+import helpers
+from oracle import partition_oracle as po
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("name", block4_codec.names())
+def test_gpu_partition_reproduces_golden(gpu, name):
+    golden = block4_codec.load(name)
+    indptr = po.indptr_from_degrees(po.degrees_from_block4(golden))
+    got = gpu.block_level_partition.partition(indptr, backend="gpu")
+    assert got.tobytes() == golden.tobytes()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_gpu_partition_on_unsorted_rows(gpu, seed):
+    """The walk also defines a result for rows that are not sorted (runs of equal
+    degree, zero-degree rows anywhere); the kernels follow it."""
+    rng = np.random.default_rng(seed)
+    deg = np.repeat(rng.choice([0, 0, 1, 2, 5, 32, 33, 64, 96, 97, 129, 191, 192, 384, 385, 768, 5000],
+                               size=700), rng.integers(1, 30, size=700))
+    indptr = po.indptr_from_degrees(deg)
+    got = gpu.block_level_partition.partition(indptr, backend="gpu")
+    assert np.array_equal(got, po.partition_closed_form(indptr))
+    assert np.array_equal(got, gpu.block_level_partition.partition(indptr, backend="host"))
+
+
+def test_stage_on_gpu_writes_golden_file(gpu, tmp_path):
+    graphs = tmp_path / "graphs"
+    graphs.mkdir()
+    for name in ("pubmed", "collab"):
+        golden = block4_codec.load(name)
+        (graphs / f"{name}.config").write_text("")
+        po.indptr_from_degrees(po.degrees_from_block4(golden)).astype("<i4").tofile(graphs / f"{name}.new_indptr")
+    done = gpu.block_level_partition.run_stage(graphs, tmp_path / "meta", verbose=False)
+    assert set(done) == {"pubmed", "collab"}
+    for name in done:
+        assert (tmp_path / "meta" / f"{name}.block4").read_bytes() == block4_codec.load(name).tobytes()
+
+
+def check_preprocess(gpu, g):
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    perm, sip, six, sval, b4 = helpers.expected_preprocess(g.indptr, g.indices, g.values)
+    assert np.array_equal(op.perm(), perm)
+    ip, ix, v = op.sorted_csr()
+    assert np.array_equal(ip, sip) and np.array_equal(ix, six) and np.array_equal(v, sval)
+    assert op.block4().tobytes() == po.block4_to_bytes(b4)
+    d = np.diff(g.indptr)
+    info = op.info
+    assert (info.rows, info.cols, info.nnz) == (g.n_rows, g.n_cols, g.nnz)
+    assert info.n_blocks == len(b4)
+    assert info.n_zero_rows == int((d == 0).sum()) and info.n_long_rows == int((d > 384).sum())
+    assert info.n_long_blocks == int(np.sum(-(-d[d > 384] // 384)))
+    assert info.max_degree == int(d.max(initial=0))
+    op.check_block4(b4)
+    return op
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_preprocess_mixed_degrees(gpu, seed):
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=seed, n_long=7, zeros=9), seed=seed)
+    op = check_preprocess(gpu, g)
+    assert op.info.already_sorted == 0
+    op.close()
+
+
+def test_preprocess_workloads(gpu):
+    for g in (gpu.synthetic.cfg1(), gpu.synthetic.cfg2(), gpu.synthetic.hub_graph_small()):
+        check_preprocess(gpu, g).close()
+
+
+def test_preprocess_needs_three_radix_passes(gpu):
+    # a degree above 65535 exercises the third 8-bit pass of the sort
+    deg = np.array([3, 70_000, 0, 3, 1, 300, 70_000, 2, 65_536, 1], dtype=np.int64)
+    g = helpers.graph_from_degrees(deg, n_cols=80_000, seed=5)
+    check_preprocess(gpu, g).close()
+
+
+def test_already_sorted_input_is_borrowed(gpu):
+    g0 = helpers.graph_from_degrees(helpers.degree_mix(seed=2), seed=2)
+    perm = po.degree_sort(g0.indptr)
+    sip, six, sval = po.permute_csr(g0.indptr, g0.indices, g0.values, perm)
+    op = gpu.AccelSpMM(sip, six, sval, g0.n_cols).preprocess()
+    assert op.info.already_sorted == 1
+    assert np.array_equal(op.perm(), np.arange(g0.n_rows))
+    assert np.array_equal(op.block4(), po.partition_closed_form(sip))
+    ip, ix, v = op.sorted_csr()
+    assert np.array_equal(ip, sip) and np.array_equal(ix, six) and np.array_equal(v, sval)
+    op.close()
+
+
+def test_edge_shapes(gpu):
+    empty = gpu.AccelSpMM(np.zeros(1, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32), 5).preprocess()
+    assert empty.info.n_blocks == 0 and empty.block4().shape == (0, 4)
+    assert empty.matmul(np.ones((5, 3), np.float32)).shape == (0, 3)
+    empty.close()
+    allzero = gpu.AccelSpMM(np.zeros(8, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32), 5).preprocess()
+    assert allzero.info.n_blocks == 0 and allzero.info.n_zero_rows == 7
+    assert np.array_equal(allzero.matmul(np.ones((5, 3), np.float32)), np.zeros((7, 3), np.float32))
+    allzero.close()
+    one = gpu.AccelSpMM(np.array([0, 2], np.int32), np.array([1, 3], np.int32),
+                        np.array([2.0, -1.0], np.float32), 4).preprocess()
+    assert one.block4().tolist() == [[2, 0, 0, (2 << 16) + 1]]
+    X = np.arange(8, dtype=np.float32).reshape(4, 2)
+    assert np.array_equal(one.matmul(X), (2 * X[1] - X[3])[None, :])
+    one.close()
+
+
+def test_bad_csr_is_rejected(gpu):
+    lib = gpu._lib
+    ok = helpers.graph_from_degrees([2, 3, 1], n_cols=6)
+    cases = {
+        "decreasing": (np.array([0, 3, 2, 6], np.int32), ok.indices, ok.values),
+        "nonzero start": (np.array([1, 2, 5, 6], np.int32), ok.indices, ok.values),
+        "wrong end": (np.array([0, 2, 4, 5], np.int32), ok.indices, ok.values),
+        "column too large": (ok.indptr, np.array([0, 1, 2, 3, 6, 0], np.int32), ok.values),
+        "negative column": (ok.indptr, np.array([0, 1, -1, 3, 4, 0], np.int32), ok.values),
+    }
+    for what, (ip, ix, v) in cases.items():
+        op = gpu.AccelSpMM(ip, ix, v, 6)
+        with pytest.raises(gpu.AccelError) as e:
+            op.preprocess()
+        assert e.value.status == lib.ERR_CSR, what
+        with pytest.raises(gpu.AccelError) as e:      # and the handle stays unusable
+            op.run(0, 0, 4)
+        assert e.value.status == lib.ERR_STATE, what
+        op.close()
+
+
+def test_stale_metadata_is_rejected(gpu):
+    g = helpers.graph_from_degrees(np.sort(helpers.degree_mix(seed=1)), seed=1)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    b4 = op.block4()
+    op.check_block4(b4)
+    bad = b4.copy()
+    bad[3, 2] += 1
+    for wrong in (bad, b4[:-1]):
+        with pytest.raises(gpu.AccelError) as e:
+            op.check_block4(wrong)
+        assert e.value.status == gpu._lib.ERR_META
+    op.close()
+
+
+def test_call_order_and_arguments(gpu):
+    g = helpers.graph_from_degrees([2, 3, 1], n_cols=6)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, 6)
+    with pytest.raises(gpu.AccelError) as e:
+        op.run(0, 0, 4)
+    assert e.value.status == gpu._lib.ERR_STATE
+    op.preprocess()
+    buf = gpu.DeviceBuffer(1024)
+    for N in (0, -3):
+        with pytest.raises(gpu.AccelError) as e:
+            op.run(buf, buf, N)
+        assert e.value.status == gpu._lib.ERR_ARG
+    with pytest.raises(gpu.AccelError) as e:
+        op.run(None, buf, 4)
+    assert e.value.status == gpu._lib.ERR_ARG
+    buf.close()
+    op.close()

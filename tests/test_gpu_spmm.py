@@ -1,0 +1,209 @@
+"""Parity of the HIP SpMM with the CPU oracle.
+
+Acceptance: max |Y - R| / max(S, tiny) <= 1e-5 with R = A X in fp64 and
+S = |A| |X| (the summation order differs from scipy's, so the error is scaled by
+the size of the terms, not of the result).  All calls go through the C ABI.
+"""
+import numpy as np
+import pytest
+
+import helpers
+from oracle import c_oracle, partition_oracle as po, spmm_oracle as so
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+ALL_N = [1, 2, 3, 4, 5, 6, 8, 12, 16, 17, 30, 32, 48, 60, 64, 100, 128, 130, 200, 256, 260, 300, 512, 515]
+
+
+@pytest.fixture(scope="module")
+def mixed(gpu):
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=7, n_long=8, zeros=11), seed=7)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    yield g, op
+    op.close()
+
+
+@pytest.mark.parametrize("N", ALL_N)
+def test_every_column_count(gpu, mixed, N):
+    """Every vector width / group width, column tails, N beyond one pass (N > 256),
+    and the N upstream's lane mapping gets wrong (130, 200)."""
+    g, op = mixed
+    X = np.random.default_rng(N).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    Y = op.matmul(X)                                   # output buffer is pre-filled with NaN
+    assert np.isfinite(Y).all(), "some row of Y was not written"
+    assert so.check(Y, g.indptr, g.indices, g.values, X) <= TOL
+    d = np.diff(g.indptr)
+    assert np.array_equal(Y[d == 0], np.zeros(((d == 0).sum(), N), np.float32))   # beta = 0
+
+
+def test_workload_cfg1(gpu):
+    g = gpu.synthetic.cfg1()
+    X = gpu.synthetic.dense_operand("cfg1", g.n_cols, 32)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    Y = op.matmul(X)
+    assert so.check(Y, g.indptr, g.indices, g.values, X) <= TOL
+    Ys = so.spmm_scipy32(g.indptr, g.indices, g.values, X)
+    assert np.max(np.abs(Y - Ys)) / np.max(np.abs(Ys)) <= TOL
+    assert so.upstream_mean_abs_error(Y, Ys) < 1e-3     # upstream's own, looser bar (main.cu:41)
+    op.close()
+
+
+@pytest.mark.parametrize("N", [16, 32, 64, 128])
+def test_workload_cfg2(gpu, N):
+    g = gpu.synthetic.cfg2()
+    X = gpu.synthetic.dense_operand("cfg2", g.n_cols, N)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    Y = op.matmul(X)
+    R, S = c_oracle.spmm_csr_f64(g.indptr, g.indices, g.values, X)
+    assert so.scaled_error(Y, R, S) <= TOL
+    op.close()
+
+
+def test_hub_rows_and_wide_X(gpu):
+    """Shape of cfg5: rows spanning several 384-non-zero segments, a majority of
+    degree-1 rows, N = 256, X ~ N(0,1), val ~ U(0,1]."""
+    g = gpu.synthetic.hub_graph_small()
+    X = gpu.synthetic.dense_operand(g.name, g.n_cols, 256)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    assert op.info.n_long_rows >= 4
+    Y = op.matmul(X)
+    assert so.check(Y, g.indptr, g.indices, g.values, X) <= TOL
+    op.close()
+
+
+def test_one_very_long_row(gpu):
+    # 100k non-zeros in one row: 261 segments reduced through the scratch buffer
+    deg = np.array([1, 100_000, 0, 2, 384, 385], dtype=np.int64)
+    g = helpers.graph_from_degrees(deg, n_cols=120_000, seed=9)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    for N in (4, 64, 100):
+        X = np.random.default_rng(N).standard_normal((g.n_cols, N)).astype(np.float32)
+        Y = op.matmul(X)
+        assert so.check(Y, g.indptr, g.indices, g.values, X) <= TOL
+    op.close()
+
+
+def test_closed_forms(gpu):
+    deg = helpers.degree_mix(seed=4, n_long=5)
+    g = helpers.graph_from_degrees(deg, seed=4, value_mode="ones")
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    Y = op.matmul(np.ones((g.n_cols, 8), np.float32))
+    assert np.array_equal(Y, np.repeat(deg[:, None], 8, 1).astype(np.float32))   # ones -> row degree, exact
+    op.close()
+    n = 777                                                                     # identity -> X, exact
+    X = np.random.default_rng(0).standard_normal((n, 20)).astype(np.float32)
+    eye = gpu.AccelSpMM(np.arange(n + 1, dtype=np.int32), np.arange(n, dtype=np.int32),
+                        np.ones(n, np.float32), n).preprocess()
+    assert np.array_equal(eye.matmul(X), X)
+    eye.close()
+
+
+def test_row_order_follows_the_callers_csr(gpu):
+    """Rows of Y are in the caller's order; the same matrix given already
+    degree-sorted (as upstream's *.new_* files are) gives the permuted rows."""
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=5, n_long=4), seed=5)
+    X = np.random.default_rng(5).uniform(-1, 1, (g.n_cols, 48)).astype(np.float32)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    Y = op.matmul(X)
+    perm = po.degree_sort(g.indptr)
+    sip, six, sval = po.permute_csr(g.indptr, g.indices, g.values, perm)
+    ops = gpu.AccelSpMM(sip, six, sval, g.n_cols).preprocess()
+    assert ops.info.already_sorted == 1
+    assert np.array_equal(ops.matmul(X), Y[perm])        # same arithmetic, same bits
+    op.close()
+    ops.close()
+
+
+def test_deterministic_and_overwrites(gpu, mixed):
+    g, op = mixed
+    X = np.random.default_rng(1).uniform(-1, 1, (g.n_cols, 64)).astype(np.float32)
+    dX = gpu.DeviceBuffer.from_numpy(X)
+    dY = gpu.DeviceBuffer(g.n_rows * 64 * 4)
+    outs = []
+    for fill in (0x7FC00000, 0x3F800000, 0):            # NaN, 1.0, 0.0 left in Y before the run
+        dY.fill_u32(fill)
+        op.run(dX, dY, 64)
+        op.run(dX, dY, 64)                               # twice: upstream would accumulate
+        op.synchronize()
+        outs.append(dY.to_numpy(np.float32, (g.n_rows, 64)))
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    assert so.check(outs[0], g.indptr, g.indices, g.values, X) <= TOL
+    dX.close()
+    dY.close()
+
+
+def test_linearity_and_column_slicing(gpu):
+    g = gpu.synthetic.cfg2()
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    rng = np.random.default_rng(2)
+    X1 = rng.uniform(-1, 1, (g.n_cols, 128)).astype(np.float32)
+    X2 = rng.uniform(-1, 1, (g.n_cols, 128)).astype(np.float32)
+    Y1, Y2, Y12 = op.matmul(X1), op.matmul(X2), op.matmul(X1 + X2)
+    scale = np.abs(Y1).max() + np.abs(Y2).max()
+    assert np.max(np.abs(Y12 - (Y1 + Y2))) <= 1e-5 * scale
+    # column j of the N=128 result is column j of the N=16 result on the same columns
+    Y16 = op.matmul(np.ascontiguousarray(X1[:, :16]))
+    assert np.max(np.abs(Y16 - Y1[:, :16])) <= 1e-5 * np.abs(Y1).max()
+    op.close()
+
+
+def test_operator_mirror_do_test(gpu, tmp_path):
+    """SpmmAccel follows SPMM_ACCEL: construct on device pointers of a
+    degree-sorted CSR, do_test(False, dim) computes, do_test(True, dim) returns
+    seconds; a matching .block4 file is accepted, a stale one refused."""
+    g0 = gpu.synthetic.cfg1()
+    perm = po.degree_sort(g0.indptr)
+    sip, six, sval = po.permute_csr(g0.indptr, g0.indices, g0.values, perm)
+    dim_max = 64
+    X = gpu.synthetic.dense_operand("cfg1", g0.n_cols, dim_max)
+    bufs = [gpu.DeviceBuffer.from_numpy(a) for a in (sip, six, sval, X)]
+    vout = gpu.DeviceBuffer(g0.n_rows * dim_max * 4)
+    meta = tmp_path / "block_level_meta"
+    meta.mkdir()
+    gpu.block_level_partition.write_block4(meta / "cfg1.block4", po.partition_closed_form(sip))
+    acc = gpu.SpmmAccel("cfg1", bufs[0], bufs[1], bufs[2], bufs[3], vout, g0.n_rows, g0.nnz, dim_max,
+                        meta_dir=meta)
+    for dim in (16, 33, 64):                              # leading dimension = current dim
+        assert acc.do_test(False, dim) == 0.0
+        Y = vout.to_numpy(np.float32, (g0.n_rows, dim))
+        Xd = X.reshape(-1)[: g0.n_cols * dim].reshape(g0.n_cols, dim)
+        assert so.check(Y, sip, six, sval, Xd) <= TOL
+    t = acc.do_test(True, 64)
+    assert 0 < t < 1.0
+    b = po.partition_closed_form(sip).copy()
+    b[0, 3] += 1
+    gpu.block_level_partition.write_block4(meta / "stale.block4", b)
+    stale = gpu.SpmmAccel("stale", bufs[0], bufs[1], bufs[2], bufs[3], vout, g0.n_rows, g0.nnz, dim_max,
+                          meta_dir=meta)
+    with pytest.raises(gpu.AccelError) as e:
+        stale.do_test(False, 16)
+    assert e.value.status == gpu._lib.ERR_META
+    for bfr in bufs + [vout]:
+        bfr.close()
+
+
+def test_timing_entry_point(gpu, mixed):
+    g, op = mixed
+    X = np.random.default_rng(3).uniform(-1, 1, (g.n_cols, 64)).astype(np.float32)
+    dX = gpu.DeviceBuffer.from_numpy(X)
+    dY = gpu.DeviceBuffer(g.n_rows * 64 * 4)
+    tot, main = op.time(dX, dY, 64, warmup=2, iters=5)
+    assert tot.shape == (5,) and np.all(tot > 0) and np.all(main > 0) and np.all(main <= tot * 1.001)
+    assert so.check(dY.to_numpy(np.float32, (g.n_rows, 64)), g.indptr, g.indices, g.values, X) <= TOL
+    dX.close()
+    dY.close()
+
+
+def test_medium_power_law_graph(gpu):
+    """A 300k-row, ~15M-edge graph generated like cfg4 (gamma 2.1)."""
+    g = gpu.synthetic.cfg4(n=300_000, n_edges=15_000_000, max_degree=17_000)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    perm, sip, six, sval, b4 = helpers.expected_preprocess(g.indptr, g.indices, g.values)
+    assert np.array_equal(op.perm(), perm) and op.block4().tobytes() == po.block4_to_bytes(b4)
+    for N in (64, 100):
+        X = gpu.synthetic.dense_operand("cfg4", g.n_cols, N)
+        Y = op.matmul(X)
+        R, S = c_oracle.spmm_csr_f64(g.indptr, g.indices, g.values, X)
+        assert so.scaled_error(Y, R, S) <= TOL
+    op.close()
