@@ -1,0 +1,164 @@
+#!/usr/bin/env python3
+"""Benchmark of the SpMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4] [--N 64]
+
+A step is one Y = A X over the whole synthetic graph, inputs resident in HBM.
+Prints ONE JSON line: GFLOP/s = 2 * nnz * N / t, the HBM-roofline figures of the
+gather kernel (algorithmic bytes = nnz*(4+4) + M*N*4 + rows*N*4 per launch,
+launch duration from HIP events recorded on the launch stream during the timed
+steps), and scipy's CSR @ dense timed on this host's cores on a bounded row
+sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_baseline(g, X, N, budget_s=15.0):
+    """scipy csr @ X (fp32, one thread) on the first rows of the CSR that fit the
+    time budget; the checker only, never the measured path."""
+    from oracle import spmm_oracle as so
+
+    rows = g.n_rows
+
+    def run(n_rows):
+        ip = g.indptr[: n_rows + 1]
+        nz = int(ip[-1])
+        A = so.csr(ip, g.indices[:nz], g.values[:nz], g.n_cols)
+        t0 = time.perf_counter()
+        Y = A @ X
+        return time.perf_counter() - t0, nz, Y
+
+    probe_rows = max(1, min(rows, rows // 50))
+    t_probe, nz_probe, _ = run(probe_rows)
+    rate = nz_probe / max(t_probe, 1e-9)                       # non-zeros per second
+    want_nz = min(g.nnz, int(rate * budget_s))
+    n_rows = int(np.searchsorted(g.indptr, want_nz, side="right")) - 1
+    n_rows = max(probe_rows, min(rows, n_rows))
+    t, nz, Y = run(n_rows)
+    return {"value": 2.0 * nz * N / t / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+            "host_cores": os.cpu_count(), "seconds": round(t, 3),
+            "sample": f"scipy.sparse csr_matrix @ dense, fp32, first {n_rows} of {rows} rows "
+                      f"({nz} of {g.nnz} non-zeros), N={N}, 1 thread"}, n_rows, Y
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--N", type=int, default=0, help="columns of X (default: the workload's first)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the scipy baseline and the check")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="only run the plain copy kernel over this many MiB, --steps times "
+                         "(known-size reference for the FETCH_SIZE / WRITE_SIZE counters)")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build measures one GPU only (the path has no multi-GPU part); "
+                 "run it with --gpus 1 in a single process")
+
+    import __graft_entry__ as entry
+    pkg = entry.load_package()
+    if pkg.device_count() < 1:
+        sys.exit("bench.py: no GPU: " + pkg._lib.last_error())
+    if a.copy_calibration:
+        import ctypes as C
+        words = a.copy_calibration * (1 << 20) // 4
+        src, dst = pkg.DeviceBuffer(words * 4), pkg.DeviceBuffer(words * 4)
+        src.fill_u32(1)
+        for _ in range(a.steps):
+            pkg._lib.check(pkg.lib().accel_dev_copy_u32(C.c_void_p(dst.address), C.c_void_p(src.address), words, None))
+        pkg._lib.check(pkg.lib().accel_stream_sync(None))
+        print(json.dumps({"copy_calibration_MiB": a.copy_calibration, "launches": a.steps,
+                          "bytes_read_per_launch": words * 4, "bytes_written_per_launch": words * 4}))
+        return
+    syn = pkg.synthetic
+    N = a.N or syn.WORKLOAD_N[a.workload][0]
+
+    t0 = time.time()
+    g = syn.WORKLOADS[a.workload]()
+    X = syn.dense_operand(a.workload, g.n_cols, N)
+    log(f"[bench] {a.workload}: rows={g.n_rows} nnz={g.nnz} N={N} generated in {time.time() - t0:.1f}s")
+
+    t0 = time.time()
+    op = pkg.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols)
+    t_upload = time.time() - t0
+    op.preprocess()
+    info = op.info
+    log(f"[bench] upload {t_upload * 1e3:.0f} ms, preprocess {info.preprocess_ms:.1f} ms: "
+        f"blocks={info.n_blocks} long_rows={info.n_long_rows} long_blocks={info.n_long_blocks} "
+        f"zero_rows={info.n_zero_rows} max_degree={info.max_degree}")
+    dX = pkg.DeviceBuffer.from_numpy(X)
+    dY = pkg.DeviceBuffer(g.n_rows * N * 4)
+    dY.fill_u32(0x7FC00000)
+
+    # warm-up, then the timed region: K steps queued back to back, bracketed by
+    # synchronisations; the events inside it give the kernel durations
+    op.time(dX, dY, N, warmup=a.warmup, iters=0)
+    op.synchronize()
+    t0 = time.perf_counter()
+    tot_ms, main_ms = op.time(dX, dY, N, warmup=0, iters=a.steps)
+    op.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / a.steps * 1e3
+
+    flops = 2.0 * g.nnz * N
+    alg_bytes = g.nnz * 8 + g.n_cols * N * 4 + g.n_rows * N * 4
+    main_avg_ms = float(np.mean(main_ms))
+    achieved = alg_bytes / (main_avg_ms * 1e-3) / 1e9
+    result = {
+        "metric": "SpMM GFLOP/s (2*nnz*N), fp32",
+        "value": round(flops / (ms_per_step * 1e-3) / 1e9, 2),
+        "unit": "GFLOP/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{a.workload}: {g.n_rows} rows, {g.nnz} non-zeros, N={N}",
+                   "rows": g.n_rows, "nnz": g.nnz, "N": N, "blocks": int(info.n_blocks),
+                   "preprocess_ms": round(info.preprocess_ms, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "spmm_gather_kernel", "kernel_ms_avg": round(main_avg_ms, 5),
+                     "kernel_ms_min": round(float(np.min(main_ms)), 5),
+                     "all_kernels_ms_avg": round(float(np.mean(tot_ms)), 5),
+                     "algorithmic_bytes": alg_bytes},
+    }
+
+    if not a.no_cpu:
+        base, n_rows, Yc = cpu_baseline(g, X, N)
+        result["cpu_baseline"] = base
+        # parity of the timed output on the baseline's rows (fp64 reference, scaled error)
+        from oracle import spmm_oracle as so
+        Y = dY.to_numpy(np.float32, (g.n_rows, N))[:n_rows]
+        nz = int(g.indptr[n_rows])
+        R, S = so.spmm_fp64(g.indptr[: n_rows + 1], g.indices[:nz], g.values[:nz], X)
+        err = so.scaled_error(Y, R, S)
+        result["parity"] = {"rows_checked": n_rows, "scaled_error": err, "tolerance": so.TOL,
+                            "ok": bool(err <= so.TOL)}
+        if err > so.TOL:
+            log(f"[bench] PARITY FAILURE: scaled error {err:.3e}")
+    print(json.dumps(result), flush=True)
+    dX.close()
+    dY.close()
+    op.close()
+    if not a.no_cpu and not result["parity"]["ok"]:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

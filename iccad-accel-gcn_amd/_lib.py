@@ -7,12 +7,14 @@ CPU stand-in for any GPU entry point.
 from __future__ import annotations
 
 import ctypes as C
+import os
 from pathlib import Path
 
 import numpy as np
 
 PKG = Path(__file__).resolve().parent
-LIB_PATH = PKG / "lib" / "libaccelgcn.so"
+# ACCEL_GCN_LIB selects another build of the same library (e.g. a tuning variant)
+LIB_PATH = Path(os.environ.get("ACCEL_GCN_LIB") or PKG / "lib" / "libaccelgcn.so")
 
 OK, ERR_ARG, ERR_CSR, ERR_ALLOC, ERR_HIP, ERR_META, ERR_STATE, ERR_IO = 0, -1, -2, -3, -4, -5, -6, -7
 PTR_HOST, PTR_DEVICE = 0, 1
@@ -59,6 +61,7 @@ SIGNATURES = {
     "accel_memcpy_h2d": (C.c_int, [vp, vp, C.c_size_t]),
     "accel_memcpy_d2h": (C.c_int, [vp, vp, C.c_size_t]),
     "accel_dev_fill_u32": (C.c_int, [vp, C.c_uint32, C.c_size_t, vp]),
+    "accel_dev_copy_u32": (C.c_int, [vp, vp, C.c_size_t, vp]),
     "accel_stream_sync": (C.c_int, [vp]),
     "accel_create": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.POINTER(vp)]),
     "accel_preprocess": (C.c_int, [vp]),

@@ -34,12 +34,16 @@ def compile_flags():
             f"-I{ROOT / 'include'}", f"-I{CSRC}"]
 
 
-def build(verbose: bool = False, extra_flags=()) -> Path:
+def build(verbose: bool = False, extra_flags=(), out: Path | None = None) -> Path:
+    """Compile and link; ``extra_flags`` (e.g. -DACCEL_UNROLL=8) and ``out`` let a
+    tuning variant be built next to the default library."""
     LIB_DIR.mkdir(exist_ok=True)
+    out = Path(out) if out else LIB
+    out.parent.mkdir(parents=True, exist_ok=True)
     objs = []
     procs = []
     for src in SOURCES:
-        obj = LIB_DIR / (src + ".o")
+        obj = out.parent / (out.stem + "." + src + ".o")
         cmd = [hipcc(), *compile_flags(), *extra_flags, "-c", str(CSRC / src), "-o", str(obj)]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -47,18 +51,20 @@ def build(verbose: bool = False, extra_flags=()) -> Path:
         objs.append(str(obj))
     failed = []
     for src, p in procs:
-        out, _ = p.communicate()
+        text, _ = p.communicate()
         if p.returncode != 0:
-            failed.append((src, out))
-        elif verbose and out.strip():
-            print(out)
+            failed.append((src, text))
+        elif verbose and text.strip():
+            print(text)
     if failed:
         raise RuntimeError("hipcc failed:\n" + "\n".join(f"--- {s}\n{o}" for s, o in failed))
-    tmp = LIB.with_suffix(".so.tmp")
+    tmp = out.with_suffix(".so.tmp")
     cmd = [hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", str(tmp)]
     subprocess.run(cmd, check=True)
-    os.replace(tmp, LIB)
-    return LIB
+    os.replace(tmp, out)
+    for o in objs:
+        os.unlink(o)
+    return out
 
 
 if __name__ == "__main__":

@@ -255,6 +255,13 @@ int accel_dev_fill_u32(void *dst, uint32_t value, size_t n_words, void *stream)
     return fill_u32(dst, value, n_words, static_cast<hipStream_t>(stream));
 }
 
+int accel_dev_copy_u32(void *dst_dev, const void *src_dev, size_t n_words, void *stream)
+{
+    clear_error();
+    if (n_words && (!dst_dev || !src_dev)) { set_error("accel_dev_copy_u32: null argument"); return ACCEL_ERR_ARG; }
+    return copy_u32(dst_dev, src_dev, n_words, static_cast<hipStream_t>(stream));
+}
+
 int accel_stream_sync(void *stream)
 {
     clear_error();
@@ -497,32 +504,31 @@ int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup,
     for (int i = 0; i < warmup; i++)
         if (int rc = spmm_launch(h, X, Y, N, s, nullptr)) return rc;
     ACCEL_HIP(hipStreamSynchronize(s));
-    hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr;
-    ACCEL_HIP(hipEventCreate(&e0));
-    ACCEL_HIP(hipEventCreate(&e1));
-    ACCEL_HIP(hipEventCreate(&e2));
+    if (iters == 0) return ACCEL_OK;
+    // all launches are queued back to back; the events are read after one final wait
+    std::vector<hipEvent_t> ev((size_t)iters * 3, nullptr);
     int rc = ACCEL_OK;
+    for (auto &e : ev)
+        if (hipEventCreate(&e) != hipSuccess) { rc = ACCEL_ERR_HIP; set_error("hipEventCreate failed"); break; }
     for (int i = 0; i < iters && !rc; i++) {
-        hipError_t e = hipEventRecord(e0, s);
-        if (e == hipSuccess) rc = spmm_launch(h, X, Y, N, s, ms_main ? e1 : nullptr);
-        if (rc) break;
-        if (e == hipSuccess) e = hipEventRecord(e2, s);
-        if (e == hipSuccess) e = hipEventSynchronize(e2);
+        hipError_t e = hipEventRecord(ev[3 * i], s);
+        if (e == hipSuccess) rc = spmm_launch(h, X, Y, N, s, ms_main ? ev[3 * i + 1] : nullptr);
+        if (!rc && e == hipSuccess) e = hipEventRecord(ev[3 * i + 2], s);
+        if (!rc && e != hipSuccess) { set_error("hipEventRecord: %s", hipGetErrorString(e)); rc = ACCEL_ERR_HIP; }
+    }
+    if (!rc && hipStreamSynchronize(s) != hipSuccess) { set_error("stream synchronisation failed"); rc = ACCEL_ERR_HIP; }
+    for (int i = 0; i < iters && !rc; i++) {
         float t = 0.f;
-        if (e == hipSuccess) e = hipEventElapsedTime(&t, e0, e2);
+        hipError_t e = hipEventElapsedTime(&t, ev[3 * i], ev[3 * i + 2]);
         if (e == hipSuccess && ms_total) ms_total[i] = t;
         if (e == hipSuccess && ms_main) {
-            e = hipEventElapsedTime(&t, e0, e1);
+            e = hipEventElapsedTime(&t, ev[3 * i], ev[3 * i + 1]);
             ms_main[i] = t;
         }
-        if (e != hipSuccess) {
-            set_error("event timing failed: %s", hipGetErrorString(e));
-            rc = ACCEL_ERR_HIP;
-        }
+        if (e != hipSuccess) { set_error("event timing failed: %s", hipGetErrorString(e)); rc = ACCEL_ERR_HIP; }
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
-    (void)hipEventDestroy(e2);
+    for (auto e : ev)
+        if (e) (void)hipEventDestroy(e);
     return rc;
 }
 

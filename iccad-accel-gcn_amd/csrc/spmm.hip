@@ -32,6 +32,28 @@ constexpr int kWaves = 4;                 // wavefronts (= block4 entries) per w
 constexpr int kWgThreads = 64 * kWaves;
 constexpr int kZeroFloats = 16384;        // floats zero-filled per extra workgroup
 
+// build-time tuning knobs (defaults are the measured best)
+#ifndef ACCEL_UNROLL
+#define ACCEL_UNROLL 4                    // gathers in flight per lane in the main loop
+#endif
+#ifndef ACCEL_NT_STREAM
+#define ACCEL_NT_STREAM 0                 // 1: read-once CSR streams bypass cache retention
+#endif
+#ifndef ACCEL_NT_STORE
+#define ACCEL_NT_STORE 0                  // 1: Y rows are stored with the non-temporal hint
+#endif
+constexpr int kUnroll = ACCEL_UNROLL;
+
+template <class T>
+__device__ __forceinline__ T stream_load(const T *p)
+{
+#if ACCEL_NT_STREAM
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
+}
+
 template <int VEC>
 __device__ __forceinline__ void load_vec(const float *__restrict__ p, float (&v)[VEC])
 {
@@ -56,6 +78,18 @@ __device__ __forceinline__ void store_vec(float *__restrict__ p, const float (&v
     } else {
         *p = v[0];
     }
+}
+
+// Y rows are written once and not read again by this launch.
+template <int VEC>
+__device__ __forceinline__ void store_out(float *__restrict__ p, const float (&v)[VEC])
+{
+#if ACCEL_NT_STORE
+#pragma unroll
+    for (int i = 0; i < VEC; i++) __builtin_nontemporal_store(v[i], p + i);
+#else
+    store_vec<VEC>(p, v);
+#endif
 }
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
@@ -107,8 +141,8 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
         for (int j = 0; j < kRounds; j++) {
             const int i = lane + 64 * j;
             if (i < total_nz) {
-                ci[j] = s_idx[loc + i];
-                cv[j] = s_val[loc + i];
+                ci[j] = stream_load(s_idx + loc + i);
+                cv[j] = stream_load(s_val + loc + i);
             }
         }
 #pragma unroll
@@ -149,15 +183,15 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
                 const int2 *row_st = st + r * d;
                 const float *xcol = X + col;
                 int o = k;
-                for (; o + 3 * gp < d; o += 4 * gp) {
-                    int2 p[4];
-                    float x[4][VEC];
+                for (; o + (kUnroll - 1) * gp < d; o += kUnroll * gp) {
+                    int2 p[kUnroll];
+                    float x[kUnroll][VEC];
 #pragma unroll
-                    for (int u = 0; u < 4; u++) p[u] = row_st[o + u * gp];
+                    for (int u = 0; u < kUnroll; u++) p[u] = row_st[o + u * gp];
 #pragma unroll
-                    for (int u = 0; u < 4; u++) load_vec<VEC>(xcol + (int64_t)p[u].x * N, x[u]);
+                    for (int u = 0; u < kUnroll; u++) load_vec<VEC>(xcol + (int64_t)p[u].x * N, x[u]);
 #pragma unroll
-                    for (int u = 0; u < 4; u++) {
+                    for (int u = 0; u < kUnroll; u++) {
                         const float a = __int_as_float(p[u].y);
 #pragma unroll
                         for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[u][v], acc[v]);
@@ -182,7 +216,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
                     store_vec<VEC>(partial + (int64_t)(e - n_short_blocks) * N + col, acc);
                 } else {
                     const int64_t out_row = perm ? perm[row0 + r] : row0 + r;
-                    store_vec<VEC>(Y + out_row * N + col, acc);
+                    store_out<VEC>(Y + out_row * N + col, acc);
                 }
             }
         }
@@ -227,6 +261,13 @@ __global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t *dst, uint32_t v
         dst[i] = v;
 }
 
+__global__ __launch_bounds__(256) void copy_u32_kernel(uint32_t *__restrict__ dst,
+                                                       const uint32_t *__restrict__ src, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+        dst[i] = src[i];
+}
+
 template <int VEC>
 int launch_for_vec(int L, dim3 grid, hipStream_t s, const int4 *block4, int n_blocks, int n_short,
                    const int32_t *s_idx, const float *s_val, const int32_t *perm, const float *X,
@@ -261,6 +302,16 @@ int fill_u32(void *dst, uint32_t v, size_t n, hipStream_t s)
     if (n == 0) return ACCEL_OK;
     const unsigned g = (unsigned)std::min<size_t>((n + 255) / 256, 4096);
     fill_u32_kernel<<<dim3(g), dim3(256), 0, s>>>(static_cast<uint32_t *>(dst), v, n);
+    ACCEL_HIP(hipGetLastError());
+    return ACCEL_OK;
+}
+
+int copy_u32(void *dst, const void *src, size_t n, hipStream_t s)
+{
+    if (n == 0) return ACCEL_OK;
+    const unsigned g = (unsigned)std::min<size_t>((n + 255) / 256, 65536);
+    copy_u32_kernel<<<dim3(g), dim3(256), 0, s>>>(static_cast<uint32_t *>(dst),
+                                                  static_cast<const uint32_t *>(src), n);
     ACCEL_HIP(hipGetLastError());
     return ACCEL_OK;
 }

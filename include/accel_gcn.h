@@ -87,6 +87,9 @@ int accel_dev_free(void *p);
 int accel_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes);
 int accel_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes);
 int accel_dev_fill_u32(void *dst_dev, uint32_t value, size_t n_words, void *stream);
+/* Plain grid-stride copy kernel of n_words 4-byte words; also the known-size
+ * reference against which hardware byte counters are calibrated. */
+int accel_dev_copy_u32(void *dst_dev, const void *src_dev, size_t n_words, void *stream);
 int accel_stream_sync(void *stream); /* NULL = default stream */
 
 /* ---- the operator ----------------------------------------------------------
