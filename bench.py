@@ -23,6 +23,17 @@ import numpy as np
 HBM_PEAK_GBS = 8000.0
 
 
+def recorded_traffic(workload, N):
+    """HBM bytes per launch from the committed rocprofv3 counter runs, if this
+    workload was profiled (the counters cannot be read from inside a timing run)."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "spmm_gather_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(f"{workload}/N{N}", {}).get("traffic_bytes")
+    except OSError:
+        return None
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -132,7 +143,8 @@ def main():
                    "rows": g.n_rows, "nnz": g.nnz, "N": N, "blocks": int(info.n_blocks),
                    "preprocess_ms": round(info.preprocess_ms, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": recorded_traffic(a.workload, N),
                      "kernel": "spmm_gather_kernel", "kernel_ms_avg": round(main_avg_ms, 5),
                      "kernel_ms_min": round(float(np.min(main_ms)), 5),
                      "all_kernels_ms_avg": round(float(np.mean(tot_ms)), 5),

@@ -34,11 +34,13 @@ static void release_products(accel_handle *h)
         if (h->s_idx) (void)hipFree(const_cast<int32_t *>(h->s_idx));
         if (h->s_val) (void)hipFree(const_cast<float *>(h->s_val));
     }
-    if (h->row_block) (void)hipFree(h->row_block);
+    if (h->work) (void)hipFree(h->work);
+    if (h->long_slot) (void)hipFree(h->long_slot);
     if (h->block4) (void)hipFree(h->block4);
     if (h->partial) (void)hipFree(h->partial);
     h->perm = nullptr; h->s_indptr = nullptr; h->s_idx = nullptr; h->s_val = nullptr;
-    h->row_block = nullptr; h->block4 = nullptr; h->partial = nullptr;
+    h->work = nullptr; h->long_slot = nullptr; h->block4 = nullptr; h->partial = nullptr;
+    h->n_units = h->n_long_units = 0;
     h->partial_floats = 0; h->owns_sorted = false; h->ready = false;
 }
 

@@ -14,6 +14,13 @@ namespace accel {
 constexpr int kDegBound = ACCEL_DEG_BOUND;            // non-zeros per block4 entry
 constexpr int kSlices = ACCEL_SLICES_PER_BLOCK;       // slices per entry (metadata ABI)
 constexpr int kSliceNz = kDegBound / kSlices;         // 32
+constexpr int kXcds = 8;                              // accelerator dies, each with its own L2
+constexpr int kWavesPerGroup = 4;                     // wavefronts (work units) per workgroup
+
+// Column group of a non-zero: which die's L2 should hold that row of X.  Eight
+// consecutive columns share a group so that neighbouring short rows of X (one
+// 128-byte line holds 8 rows at N = 4) stay together.
+__host__ __device__ inline int col_group(int c) { return (c >> 3) & (kXcds - 1); }
 
 // last-error string of the calling thread
 void set_error(const char *fmt, ...);
@@ -59,8 +66,12 @@ struct accel_handle {
     const int32_t *s_idx = nullptr;   // [nnz]  (aliases idx when identity)
     const float *s_val = nullptr;     // [nnz]  (aliases val when identity)
     bool owns_sorted = false;
-    int32_t *row_block = nullptr;     // [rows+1] first block4 entry of each sorted row
-    int32_t *block4 = nullptr;        // [4*n_blocks]
+    int32_t *block4 = nullptr;        // [4*n_blocks]  the .block4 metadata (upstream ABI)
+    // launch plan derived from block4 (see preprocess.hip, "work list")
+    int32_t *work = nullptr;          // [4*n_units] one int4 per wavefront
+    int64_t n_units = 0;              // multiple of 4 * kXcds
+    int64_t n_long_units = 0;         // units that write a partial sum
+    int32_t *long_slot = nullptr;     // [n_long_rows+1] partial-sum slots of each long row
     int64_t n_blocks = 0, n_long_blocks = 0, n_long_rows = 0, n_zero_rows = 0;
     int32_t max_degree = 0;
     double preprocess_ms = 0.0;

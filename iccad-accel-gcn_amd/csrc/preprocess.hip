@@ -284,19 +284,83 @@ __global__ __launch_bounds__(kThreads) void iota_kernel(uint32_t *out, int64_t n
 __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
     const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
     const float *__restrict__ val, const int32_t *__restrict__ perm,
-    const int32_t *__restrict__ s_indptr, int64_t rows, int64_t nnz, int32_t *__restrict__ s_idx,
+    const int32_t *__restrict__ s_indptr, int64_t rows, int64_t n_take, int32_t *__restrict__ s_idx,
     float *__restrict__ s_val)
 {
     const int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    if (p >= nnz) return;
+    if (p >= n_take) return;
     int64_t lo = 0, hi = rows - 1;  // first row whose end is beyond p
     while (lo < hi) {
         const int64_t mid = (lo + hi) >> 1;
         if ((int64_t)s_indptr[mid + 1] > p) hi = mid; else lo = mid + 1;
     }
-    const int64_t src = (int64_t)indptr[perm[lo]] + (p - s_indptr[lo]);
+    const int64_t src = (int64_t)indptr[perm ? perm[lo] : lo] + (p - s_indptr[lo]);
     s_idx[p] = idx[src];
     s_val[p] = val[src];
+}
+
+// ---------------------------------------------------------------------------
+// Long rows (more than 384 non-zeros): the row's non-zeros are written to the
+// sorted CSR grouped by col_group(column), stably inside each group, so that a
+// work unit of such a row touches rows of X that belong to one die's share.
+// One workgroup per long row; counts[lr*8 + g] receives the size of each group.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
+    const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
+    const float *__restrict__ val, const int32_t *__restrict__ perm,
+    const int32_t *__restrict__ s_indptr, int64_t first_long_row, int32_t *__restrict__ s_idx,
+    float *__restrict__ s_val, int *__restrict__ counts)
+{
+    __shared__ int cnt[kXcds];
+    __shared__ int base[kXcds];
+    __shared__ int wave_cnt[2][kThreads / 64][kXcds];
+    const int64_t r = first_long_row + blockIdx.x;
+    const int64_t src0 = indptr[perm ? perm[r] : r];
+    const int64_t dst0 = s_indptr[r];
+    const int d = s_indptr[r + 1] - s_indptr[r];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (threadIdx.x < kXcds) cnt[threadIdx.x] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < d; i += kThreads) atomicAdd(&cnt[col_group(idx[src0 + i])], 1);
+    __syncthreads();
+    if (threadIdx.x < kXcds) {
+        int b = 0;
+        for (int g = 0; g < (int)threadIdx.x; g++) b += cnt[g];
+        base[threadIdx.x] = b;
+        counts[(int64_t)blockIdx.x * kXcds + threadIdx.x] = cnt[threadIdx.x];
+    }
+    __syncthreads();
+    int flip = 0;
+    for (int c0 = 0; c0 < d; c0 += kThreads, flip ^= 1) {
+        const int i = c0 + threadIdx.x;
+        const bool valid = i < d;
+        const int col = valid ? idx[src0 + i] : 0;
+        const float v = valid ? val[src0 + i] : 0.0f;
+        const int g = col_group(col);
+        int rank = 0;
+#pragma unroll
+        for (int gg = 0; gg < kXcds; gg++) {
+            const unsigned long long m = __ballot(valid && g == gg);
+            if (g == gg) rank = __popcll(m & ((1ull << lane) - 1ull));
+            if (lane == 0) wave_cnt[flip][w][gg] = __popcll(m);
+        }
+        __syncthreads();
+        if (valid) {
+            int pos = base[g] + rank;
+            for (int q = 0; q < w; q++) pos += wave_cnt[flip][q][g];
+            s_idx[dst0 + pos] = col;
+            s_val[dst0 + pos] = v;
+        }
+        __syncthreads();
+        if (threadIdx.x < kXcds) {
+            int add = 0;
+#pragma unroll
+            for (int q = 0; q < kThreads / 64; q++) add += wave_cnt[flip][q][threadIdx.x];
+            base[threadIdx.x] += add;
+        }
+        // the next round writes the other half of wave_cnt and reads base only
+        // after its own barrier, so no third barrier is needed here
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -374,11 +438,10 @@ inline unsigned grid_for(int64_t n) { return (unsigned)((n + kThreads - 1) / kTh
 
 }  // namespace
 
-// Builds row_block[rows+1] and block4 from degrees given in partition order.
-// Outputs are freshly allocated device arrays (caller frees).  *n_blocks on host.
+// Builds block4 from degrees given in partition order.  The output is a freshly
+// allocated device array (caller frees); *n_blocks is returned on the host.
 static int partition_device(const uint32_t *deg, const int32_t *s_indptr, int64_t rows,
-                            int32_t **row_block_out, int32_t **block4_out, int64_t *n_blocks,
-                            hipStream_t s)
+                            int32_t **block4_out, int64_t *n_blocks, hipStream_t s)
 {
     DevBuf head, cnt, sums, rb, b4;
     int rc;
@@ -404,7 +467,6 @@ static int partition_device(const uint32_t *deg, const int32_t *s_indptr, int64_
     ACCEL_HIP(hipGetLastError());
     ACCEL_HIP(hipStreamSynchronize(s));
     *n_blocks = nb;
-    *row_block_out = static_cast<int32_t *>(rb.release());
     *block4_out = static_cast<int32_t *>(b4.release());
     return ACCEL_OK;
 }
@@ -429,10 +491,84 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
         set_error("indptr must start at 0, be non-decreasing and end at nnz");
         return ACCEL_ERR_CSR;
     }
-    int32_t *rb = nullptr;
-    rc = partition_device(deg.as<uint32_t>(), indptr_dev, rows, &rb, block4_dev, n_blocks, s);
-    if (rb) (void)hipFree(rb);
-    return rc;
+    return partition_device(deg.as<uint32_t>(), indptr_dev, rows, block4_dev, n_blocks, s);
+}
+
+// The launch plan.  One work unit per wavefront, kWavesPerGroup units per
+// workgroup, as int4 (x, y, z, w):
+//   x <= 384 : a block4 entry for whole rows, copied verbatim (degree, first
+//              row, first non-zero, (w_nz << 16) + n_rows);
+//   x  > 384 : a piece of a long row: partial-sum slot x - 385, row y, first
+//              non-zero z, length w <= 384, all of one column group;
+//   w == 0   : padding, nothing to do.
+// Workgroups are dispatched to the eight dies round-robin (workgroup i runs on
+// die i % 8), so the list is laid out as eight interleaved queues: units of
+// column group g of the long rows go to queue g, whose die then keeps that
+// share of X in its own L2; block4 entries of short rows fill all queues
+// evenly.  Every queue runs its heaviest units first.
+static int build_work_list(accel_handle *h, const std::vector<int32_t> &long_ptr,
+                           const std::vector<int> &group_count, int64_t first_long, hipStream_t s)
+{
+    struct Unit { int32_t x, y, z, w; };
+    const int64_t n_long = (int64_t)long_ptr.size() - 1;
+    const int64_t n_short = h->n_blocks - h->n_long_blocks;
+    std::vector<Unit> short_units((size_t)n_short);
+    if (n_short > 0)
+        ACCEL_HIP(hipMemcpyAsync(short_units.data(), h->block4, sizeof(Unit) * (size_t)n_short,
+                                 hipMemcpyDeviceToHost, s));
+    // partial-sum slots: contiguous per long row, in row order
+    std::vector<int32_t> slot((size_t)n_long + 1, 0);
+    for (int64_t lr = 0; lr < n_long; lr++) {
+        int u = 0;
+        for (int g = 0; g < kXcds; g++) u += (group_count[(size_t)lr * kXcds + g] + kDegBound - 1) / kDegBound;
+        slot[(size_t)lr + 1] = slot[(size_t)lr] + u;
+    }
+    const int64_t n_long_units = slot[(size_t)n_long];
+    std::vector<Unit> queue[kXcds];
+    for (int64_t lr = n_long - 1; lr >= 0; lr--) {      // largest rows first
+        int32_t at = long_ptr[(size_t)lr], sl = slot[(size_t)lr];
+        for (int g = 0; g < kXcds; g++) {
+            const int c = group_count[(size_t)lr * kXcds + g];
+            for (int off = 0; off < c; off += kDegBound)
+                queue[g].push_back(Unit{kDegBound + 1 + sl++, (int32_t)(first_long + lr), at + off,
+                                        std::min(kDegBound, c - off)});
+            at += c;
+        }
+    }
+    ACCEL_HIP(hipStreamSynchronize(s));
+    size_t longest = 0;
+    for (auto &q : queue) longest = std::max(longest, q.size());
+    const size_t total = (size_t)n_long_units + (size_t)n_short;
+    size_t per_queue = std::max(longest, (total + kXcds - 1) / kXcds);
+    per_queue = (per_queue + kWavesPerGroup - 1) / kWavesPerGroup * kWavesPerGroup;
+    // short entries, highest degree first, dealt to the queues that still have room
+    {
+        int g = 0;
+        for (int64_t e = n_short - 1; e >= 0; e--) {
+            int tries = 0;
+            while (queue[g].size() >= per_queue && tries < kXcds) { g = (g + 1) % kXcds; tries++; }
+            queue[g].push_back(short_units[(size_t)e]);
+            g = (g + 1) % kXcds;
+        }
+    }
+    for (auto &q : queue) q.resize(per_queue, Unit{0, 0, 0, 0});
+    std::vector<Unit> work(per_queue * kXcds);
+    for (size_t q = 0; q < per_queue / kWavesPerGroup; q++)
+        for (int g = 0; g < kXcds; g++)
+            for (int w = 0; w < kWavesPerGroup; w++)
+                work[(q * kXcds + g) * kWavesPerGroup + w] = queue[g][q * kWavesPerGroup + w];
+    h->n_units = (int64_t)work.size();
+    h->n_long_units = n_long_units;
+    DevBuf dwork, dslot;
+    int rc;
+    if ((rc = dwork.alloc(sizeof(Unit) * work.size()))) return rc;
+    if ((rc = dslot.alloc(sizeof(int32_t) * slot.size()))) return rc;
+    if (!work.empty())
+        ACCEL_HIP(hipMemcpy(dwork.p, work.data(), sizeof(Unit) * work.size(), hipMemcpyHostToDevice));
+    ACCEL_HIP(hipMemcpy(dslot.p, slot.data(), sizeof(int32_t) * slot.size(), hipMemcpyHostToDevice));
+    h->work = static_cast<int32_t *>(dwork.release());
+    h->long_slot = static_cast<int32_t *>(dslot.release());
+    return ACCEL_OK;
 }
 
 int preprocess_device(accel_handle *h)
@@ -445,6 +581,7 @@ int preprocess_device(accel_handle *h)
     h->ready = false;
     h->n_blocks = h->n_long_blocks = h->n_long_rows = h->n_zero_rows = 0;
     h->max_degree = 0;
+    h->n_units = h->n_long_units = 0;
     if (rows == 0) {
         h->identity_perm = true;
         h->ready = true;
@@ -520,38 +657,69 @@ int preprocess_device(accel_handle *h)
                                         sip.as<int>() + rows, ssums.as<int>(), s)))
         return rc;
 
-    // ---- permuted CSR -------------------------------------------------------
-    DevBuf sidx, sval, permbuf;
-    if (!h->identity_perm) {
+    // ---- sorted CSR ---------------------------------------------------------
+    // Rows of degree <= 384 keep their non-zero order; long rows are grouped by
+    // column group.  The caller's arrays are used in place only when the input
+    // was already sorted and has no long row.
+    const int64_t n_long = hs.n_long_rows, first_long = rows - n_long;
+    std::vector<int32_t> long_ptr((size_t)n_long + 1);   // s_indptr[first_long .. rows]
+    ACCEL_HIP(hipMemcpyAsync(long_ptr.data(), sip.as<int32_t>() + first_long,
+                             sizeof(int32_t) * long_ptr.size(), hipMemcpyDeviceToHost, s));
+    ACCEL_HIP(hipStreamSynchronize(s));
+    const int64_t nnz_short = long_ptr[0];
+    const bool own_copy = !h->identity_perm || n_long > 0;
+    DevBuf sidx, sval, permbuf, gcount;
+    std::vector<int> group_count((size_t)n_long * kXcds);
+    if (own_copy) {
         if ((rc = sidx.alloc(sizeof(int32_t) * (size_t)nnz))) return rc;
         if ((rc = sval.alloc(sizeof(float) * (size_t)nnz))) return rc;
-        if (nnz > 0)
-            permute_csr_kernel<<<dim3(grid_for(nnz)), dim3(kThreads), 0, s>>>(
-                h->indptr, h->idx, h->val, reinterpret_cast<const int32_t *>(perm), sip.as<int32_t>(),
-                rows, nnz, sidx.as<int32_t>(), sval.as<float>());
-        if ((rc = permbuf.alloc(sizeof(int32_t) * (size_t)rows))) return rc;
-        ACCEL_HIP(hipMemcpyAsync(permbuf.p, perm, sizeof(int32_t) * (size_t)rows,
-                                 hipMemcpyDeviceToDevice, s));
+        const int32_t *pm = reinterpret_cast<const int32_t *>(perm);
+        if (h->identity_perm) {
+            if (nnz_short > 0) {
+                ACCEL_HIP(hipMemcpyAsync(sidx.p, h->idx, sizeof(int32_t) * (size_t)nnz_short,
+                                         hipMemcpyDeviceToDevice, s));
+                ACCEL_HIP(hipMemcpyAsync(sval.p, h->val, sizeof(float) * (size_t)nnz_short,
+                                         hipMemcpyDeviceToDevice, s));
+            }
+        } else {
+            if (nnz_short > 0)
+                permute_csr_kernel<<<dim3(grid_for(nnz_short)), dim3(kThreads), 0, s>>>(
+                    h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), rows, nnz_short,
+                    sidx.as<int32_t>(), sval.as<float>());
+            if ((rc = permbuf.alloc(sizeof(int32_t) * (size_t)rows))) return rc;
+            ACCEL_HIP(hipMemcpyAsync(permbuf.p, perm, sizeof(int32_t) * (size_t)rows,
+                                     hipMemcpyDeviceToDevice, s));
+        }
+        if (n_long > 0) {
+            if ((rc = gcount.alloc(sizeof(int) * group_count.size()))) return rc;
+            group_long_rows_kernel<<<dim3((unsigned)n_long), dim3(kThreads), 0, s>>>(
+                h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), first_long, sidx.as<int32_t>(),
+                sval.as<float>(), gcount.as<int>());
+            ACCEL_HIP(hipMemcpyAsync(group_count.data(), gcount.p, sizeof(int) * group_count.size(),
+                                     hipMemcpyDeviceToHost, s));
+        }
         ACCEL_HIP(hipGetLastError());
     }
 
     // ---- partition ----------------------------------------------------------
-    int32_t *rb = nullptr, *b4 = nullptr;
+    int32_t *b4 = nullptr;
     int64_t nb = 0;
-    if ((rc = partition_device(sdeg, sip.as<int32_t>(), rows, &rb, &b4, &nb, s))) return rc;
+    if ((rc = partition_device(sdeg, sip.as<int32_t>(), rows, &b4, &nb, s))) return rc;
     ACCEL_HIP(hipStreamSynchronize(s));
-
-    h->row_block = rb;
     h->block4 = b4;
     h->n_blocks = nb;
+
+    // ---- work list ------------------------------------------------------------
+    if ((rc = build_work_list(h, long_ptr, group_count, first_long, s))) return rc;
+
     h->s_indptr = static_cast<int32_t *>(sip.release());
-    if (h->identity_perm) {
+    if (!own_copy) {
         h->perm = nullptr;
         h->s_idx = h->idx;
         h->s_val = h->val;
         h->owns_sorted = false;
     } else {
-        h->perm = static_cast<int32_t *>(permbuf.release());
+        h->perm = static_cast<int32_t *>(permbuf.release());   // stays null for sorted input
         h->s_idx = static_cast<int32_t *>(sidx.release());
         h->s_val = static_cast<float *>(sval.release());
         h->owns_sorted = true;

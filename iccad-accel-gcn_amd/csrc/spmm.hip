@@ -1,25 +1,27 @@
 // The SpMM gather kernel for gfx950 (wave64) and its two helpers.
 //
-// Work decomposition.  The unit of work is one block4 entry (upstream's
-// spmm_accel.cu:18-28 gives one CUDA thread block of 12 32-lane warps to each
-// entry); here one 64-lane wavefront takes one entry and a 256-thread workgroup
-// takes four consecutive entries.  An entry is either up to 12 whole rows of one
-// degree (<= 384 non-zeros in total) or one <= 384-non-zero segment of a row with
-// more than 384 non-zeros.
+// Work decomposition.  Upstream gives one CUDA thread block of 12 32-lane warps
+// to each block4 entry (spmm_accel.cu:18-28).  Here one 64-lane wavefront takes
+// one work unit and a 256-thread workgroup takes four.  A unit is either a
+// block4 entry of whole rows (up to 12 rows of one degree, <= 384 non-zeros in
+// total) or a piece of <= 384 non-zeros of a row with more than 384 non-zeros.
+// The units come from a launch plan built by the preprocessing step; it orders
+// them so that workgroup i, which the hardware places on die i % 8, works on
+// the column group (share of X) that die keeps in its own L2.
 //
 // Inside the wavefront the lanes form G = 64 / L groups of L lanes; a group owns
 // L * VEC consecutive columns of X/Y (VEC = 4 floats = one 16-byte load per lane
 // when N allows), so one vector-memory instruction gathers G different rows of X.
 // This replaces upstream's "combined warp" of ceil32(N) lanes that walks one
 // non-zero at a time with 4-byte loads (spmm_accel.cu:37-48,56-78).  G groups are
-// split over the entry's rows as gp groups per row (gp a power of two chosen per
-// entry to minimise the step count); the gp partial sums of a row are combined by
+// split over the unit's rows as gp groups per row (gp a power of two chosen per
+// unit to minimise the step count); the gp partial sums of a row are combined by
 // a cross-lane butterfly, so short rows need no atomics (upstream: atomicAdd for
 // every row that spans more than one warp, spmm_accel.cu:82-99).
 //
-// The (column index, value) pairs of the entry are first staged in LDS with
+// The (column index, value) pairs of the unit are first staged in LDS with
 // coalesced loads, one pair per lane; each group then reads its pairs back with
-// broadcast LDS reads.  Segments of long rows write their partial sums to a
+// broadcast LDS reads.  Pieces of long rows write their partial sums to a
 // scratch buffer and a second small kernel adds them up in a fixed order, so the
 // result is run-to-run deterministic.  Rows of degree 0 are zero-filled by extra
 // workgroups of the same launch: Y = A X holds after every run with no memset.
@@ -28,7 +30,7 @@
 namespace accel {
 namespace {
 
-constexpr int kWaves = 4;                 // wavefronts (= block4 entries) per workgroup
+constexpr int kWaves = kWavesPerGroup;    // wavefronts (= work units) per workgroup
 constexpr int kWgThreads = 64 * kWaves;
 constexpr int kZeroFloats = 16384;        // floats zero-filled per extra workgroup
 
@@ -96,7 +98,7 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 
 template <int L, int VEC>
 __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
-    const int4 *__restrict__ block4, int n_blocks, int n_short_blocks,
+    const int4 *__restrict__ work, int n_units,
     const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
     const int32_t *__restrict__ perm, const float *__restrict__ X, float *__restrict__ Y,
     float *__restrict__ partial, int N, int n_zero_rows, int n_entry_groups)
@@ -120,12 +122,12 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 
     const int lane = threadIdx.x & 63;
     const int wv = uniform(threadIdx.x >> 6);
-    int e = (int)blockIdx.x * kWaves + wv;
-    if (e >= n_blocks) return;
-    e = n_blocks - 1 - e;            // heaviest entries (long-row segments) are scheduled first
+    const int e = (int)blockIdx.x * kWaves + wv;
+    if (e >= n_units) return;
 
-    const int4 b = block4[e];
+    const int4 b = work[e];
     const int deg = uniform(b.x), row0 = uniform(b.y), loc = uniform(b.z), info = uniform(b.w);
+    if (info == 0) return;                              // padding unit
     const bool is_long = deg > kDegBound;
     const int n_rows = is_long ? 1 : (info & 0xFFFF);   // spmm_accel.cu:26
     const int d = is_long ? info : deg;                 // spmm_accel.cu:28: non-zeros per row here
@@ -213,7 +215,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
             }
             if (live && k == 0) {
                 if (is_long) {
-                    store_vec<VEC>(partial + (int64_t)(e - n_short_blocks) * N + col, acc);
+                    store_vec<VEC>(partial + (int64_t)(deg - (kDegBound + 1)) * N + col, acc);
                 } else {
                     const int64_t out_row = perm ? perm[row0 + r] : row0 + r;
                     store_out<VEC>(Y + out_row * N + col, acc);
@@ -223,21 +225,20 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     }
 }
 
-// Adds the segment partials of each long row in segment order and writes the row.
+// Adds the partial sums of each long row in slot order and writes the row.
 __global__ __launch_bounds__(kWgThreads) void long_row_reduce_kernel(
-    const float *__restrict__ partial, const int32_t *__restrict__ s_indptr,
-    const int32_t *__restrict__ row_block, const int32_t *__restrict__ perm, int64_t first_long_row,
-    int n_short_blocks, float *__restrict__ Y, int N)
+    const float *__restrict__ partial, const int32_t *__restrict__ long_slot,
+    const int32_t *__restrict__ perm, int64_t first_long_row, float *__restrict__ Y, int N)
 {
     __shared__ float red[kWgThreads];
     const int64_t r = first_long_row + blockIdx.x;
-    const int d = s_indptr[r + 1] - s_indptr[r];
-    const int nseg = (d + kDegBound - 1) / kDegBound;
-    const float *src = partial + (int64_t)(row_block[r] - n_short_blocks) * N;
+    const int first = long_slot[blockIdx.x];
+    const int nseg = long_slot[blockIdx.x + 1] - first;
+    const float *src = partial + (int64_t)first * N;
     const int64_t out_row = perm ? perm[r] : r;
     int cw = 1;                                   // columns per pass: power of two <= 256
     while (cw < N && cw < kWgThreads) cw <<= 1;
-    const int sg = kWgThreads / cw;               // segment groups
+    const int sg = kWgThreads / cw;               // slot groups
     const int c_in = threadIdx.x % cw, my_sg = threadIdx.x / cw;
     for (int c0 = 0; c0 < N; c0 += cw) {
         const int c = c0 + c_in;
@@ -269,14 +270,14 @@ __global__ __launch_bounds__(256) void copy_u32_kernel(uint32_t *__restrict__ ds
 }
 
 template <int VEC>
-int launch_for_vec(int L, dim3 grid, hipStream_t s, const int4 *block4, int n_blocks, int n_short,
+int launch_for_vec(int L, dim3 grid, hipStream_t s, const int4 *work, int n_units,
                    const int32_t *s_idx, const float *s_val, const int32_t *perm, const float *X,
                    float *Y, float *partial, int N, int n_zero_rows, int n_entry_groups)
 {
 #define ACCEL_LAUNCH(LL)                                                                      \
     case LL:                                                                                  \
         spmm_gather_kernel<LL, VEC><<<grid, dim3(kWgThreads), 0, s>>>(                        \
-            block4, n_blocks, n_short, s_idx, s_val, perm, X, Y, partial, N, n_zero_rows,     \
+            work, n_units, s_idx, s_val, perm, X, Y, partial, N, n_zero_rows,                 \
             n_entry_groups);                                                                  \
         break;
     switch (L) {
@@ -328,9 +329,8 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     int L = 1;
     while (L * vec < N && L < 64) L <<= 1;
 
-    const int64_t n_short = h->n_blocks - h->n_long_blocks;
-    if (h->n_long_blocks > 0) {
-        const size_t need = (size_t)h->n_long_blocks * (size_t)N;
+    if (h->n_long_units > 0) {
+        const size_t need = (size_t)h->n_long_units * (size_t)N;
         if (h->partial_floats < need) {
             if (h->partial) (void)hipFree(h->partial);
             h->partial = nullptr;
@@ -344,7 +344,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
             h->partial_floats = need;
         }
     }
-    const int64_t entry_groups = (h->n_blocks + kWaves - 1) / kWaves;
+    const int64_t entry_groups = h->n_units / kWaves;
     const int64_t zero_groups = (h->n_zero_rows * (int64_t)N + kZeroFloats - 1) / kZeroFloats;
     const int64_t groups = entry_groups + zero_groups;
     if (groups > 0x7fffffffLL) {
@@ -354,26 +354,22 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     int rc = ACCEL_OK;
     if (groups > 0) {
         const dim3 grid((unsigned)groups);
-        const int4 *b4 = reinterpret_cast<const int4 *>(h->block4);
+        const int4 *wk = reinterpret_cast<const int4 *>(h->work);
         if (vec == 4)
-            rc = launch_for_vec<4>(L, grid, stream, b4, (int)h->n_blocks, (int)n_short, h->s_idx,
-                                   h->s_val, h->perm, X, Y, h->partial, N, (int)h->n_zero_rows,
-                                   (int)entry_groups);
+            rc = launch_for_vec<4>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
+                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups);
         else if (vec == 2)
-            rc = launch_for_vec<2>(L, grid, stream, b4, (int)h->n_blocks, (int)n_short, h->s_idx,
-                                   h->s_val, h->perm, X, Y, h->partial, N, (int)h->n_zero_rows,
-                                   (int)entry_groups);
+            rc = launch_for_vec<2>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
+                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups);
         else
-            rc = launch_for_vec<1>(L, grid, stream, b4, (int)h->n_blocks, (int)n_short, h->s_idx,
-                                   h->s_val, h->perm, X, Y, h->partial, N, (int)h->n_zero_rows,
-                                   (int)entry_groups);
+            rc = launch_for_vec<1>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
+                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups);
         if (rc) return rc;
     }
     if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));
     if (h->n_long_rows > 0) {
         long_row_reduce_kernel<<<dim3((unsigned)h->n_long_rows), dim3(kWgThreads), 0, stream>>>(
-            h->partial, h->s_indptr, h->row_block, h->perm, h->rows - h->n_long_rows, (int)n_short,
-            Y, N);
+            h->partial, h->long_slot, h->perm, h->rows - h->n_long_rows, Y, N);
     }
     ACCEL_HIP(hipGetLastError());
     return ACCEL_OK;

@@ -201,6 +201,33 @@ def permute_csr(indptr, indices, values, perm):
             None if values is None else np.asarray(values)[src])
 
 
+N_COLUMN_GROUPS = 8
+
+
+def column_group(col):
+    """Which of the 8 column groups a column belongs to (groups of 8 consecutive
+    columns, round-robin).  This is the build's own layout rule for rows with
+    more than 384 non-zeros; upstream has no counterpart (it never reorders the
+    non-zeros of a row), so it is pinned by its definition and by the SpMM
+    result being unchanged."""
+    return (np.asarray(col) >> 3) & (N_COLUMN_GROUPS - 1)
+
+
+def group_long_rows(indptr, indices, values):
+    """Stable partition of the non-zeros of every row with degree > 384 by
+    column_group(); all other rows are left as they are."""
+    indptr = np.asarray(indptr, dtype=np.int64)
+    indices = np.array(indices, copy=True)
+    values = None if values is None else np.array(values, copy=True)
+    for r in np.flatnonzero(np.diff(indptr) > DEG_BOUND):
+        a, b = indptr[r], indptr[r + 1]
+        order = np.argsort(column_group(indices[a:b]), kind="stable")
+        indices[a:b] = indices[a:b][order]
+        if values is not None:
+            values[a:b] = values[a:b][order]
+    return indices, values
+
+
 def block4_to_bytes(block4):
     """Raw little-endian int32, [deg,row,loc,info] interleaved per block
     (block_level_partition.py:105-106)."""

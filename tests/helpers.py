@@ -40,4 +40,5 @@ def expected_preprocess(indptr, indices, values):
     """(perm, sorted indptr/indices/values, block4) from the CPU oracle."""
     perm = po.degree_sort(indptr)
     sip, six, sval = po.permute_csr(indptr, indices, values, perm)
+    six, sval = po.group_long_rows(sip, six, sval)       # long rows: grouped by column group
     return perm, sip, six, sval, po.partition_closed_form(sip)

@@ -84,16 +84,20 @@ def test_preprocess_needs_three_radix_passes(gpu):
     check_preprocess(gpu, g).close()
 
 
-def test_already_sorted_input_is_borrowed(gpu):
-    g0 = helpers.graph_from_degrees(helpers.degree_mix(seed=2), seed=2)
+@pytest.mark.parametrize("n_long", [0, 4])
+def test_already_sorted_input(gpu, n_long):
+    """Input in upstream's *.new_* order: the sort is skipped, perm is the
+    identity, and only rows with more than 384 non-zeros are regrouped."""
+    g0 = helpers.graph_from_degrees(helpers.degree_mix(seed=2, n_long=n_long), seed=2)
     perm = po.degree_sort(g0.indptr)
     sip, six, sval = po.permute_csr(g0.indptr, g0.indices, g0.values, perm)
     op = gpu.AccelSpMM(sip, six, sval, g0.n_cols).preprocess()
-    assert op.info.already_sorted == 1
+    assert op.info.already_sorted == 1 and op.info.n_long_rows == n_long
     assert np.array_equal(op.perm(), np.arange(g0.n_rows))
     assert np.array_equal(op.block4(), po.partition_closed_form(sip))
     ip, ix, v = op.sorted_csr()
-    assert np.array_equal(ip, sip) and np.array_equal(ix, six) and np.array_equal(v, sval)
+    gix, gval = po.group_long_rows(sip, six, sval)
+    assert np.array_equal(ip, sip) and np.array_equal(ix, gix) and np.array_equal(v, gval)
     op.close()
 
 

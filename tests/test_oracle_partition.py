@@ -150,3 +150,23 @@ def test_permute_csr_moves_whole_rows():
     for new, old in enumerate(perm):
         assert np.array_equal(six[sip[new]:sip[new + 1]], idx[indptr[old]:indptr[old + 1]])
         assert np.array_equal(sval[sip[new]:sip[new + 1]], val[indptr[old]:indptr[old + 1]])
+
+
+def test_group_long_rows_is_a_stable_partition():
+    rng = np.random.default_rng(1)
+    deg = np.array([5, 400, 384, 1000, 0, 385])
+    indptr = po.indptr_from_degrees(deg)
+    idx = rng.integers(0, 5000, size=int(indptr[-1])).astype(np.int32)
+    val = rng.random(idx.size).astype(np.float32)
+    gi, gv = po.group_long_rows(indptr, idx, val)
+    for r, d in enumerate(deg):
+        a, b = indptr[r], indptr[r + 1]
+        if d <= 384:
+            assert np.array_equal(gi[a:b], idx[a:b]) and np.array_equal(gv[a:b], val[a:b])
+            continue
+        grp = po.column_group(gi[a:b])
+        assert np.all(np.diff(grp) >= 0)                          # grouped
+        for g in range(8):                                        # original order inside a group
+            assert np.array_equal(gi[a:b][grp == g], idx[a:b][po.column_group(idx[a:b]) == g])
+        assert sorted(zip(gi[a:b].tolist(), gv[a:b].tolist())) == sorted(zip(idx[a:b].tolist(), val[a:b].tolist()))
+    assert po.column_group(np.array([0, 7, 8, 15, 16, 63, 64])).tolist() == [0, 0, 1, 1, 2, 7, 0]
