@@ -16,6 +16,7 @@ ROOT = PKG.parent
 CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB = LIB_DIR / "libaccelgcn.so"
+BIN_DIR = PKG / "bin"
 SOURCES = ["capi.hip", "preprocess.hip", "spmm.hip", "spmm_accel.cpp"]
 ARCH = "gfx950"
 
@@ -64,7 +65,23 @@ def build(verbose: bool = False, extra_flags=(), out: Path | None = None) -> Pat
     os.replace(tmp, out)
     for o in objs:
         os.unlink(o)
+    if out == LIB:
+        build_cli(verbose)
     return out
+
+
+def build_cli(verbose: bool = False) -> Path:
+    """bin/spmm_test: the command-line harness (counterpart of upstream's main.cu)."""
+    BIN_DIR.mkdir(exist_ok=True)
+    exe = BIN_DIR / "spmm_test"
+    cmd = [hipcc(), *compile_flags(), str(CSRC / "spmm_test.cpp"), "-o", str(exe),
+           f"-L{LIB_DIR}", "-laccelgcn", "-Wl,-rpath,$ORIGIN/../lib"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for spmm_test.cpp:\n" + r.stdout)
+    return exe
 
 
 if __name__ == "__main__":

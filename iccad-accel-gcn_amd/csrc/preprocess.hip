@@ -158,37 +158,49 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
                                                           uint32_t *__restrict__ deg,
                                                           Stats *__restrict__ st)
 {
-    const int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    int bad = 0, unsorted = 0, d = 0, zero = 0, lrow = 0, lblk = 0;
-    if (r < rows) {
+    // grid-stride over rows; one set of atomics per workgroup
+    __shared__ int part[kThreads / 64][6];
+    int bad = 0, unsorted = 0, dmax = 0, zero = 0, lrow = 0, lblk = 0;
+    for (int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x; r < rows;
+         r += (int64_t)gridDim.x * kThreads) {
         const int a = indptr[r], b = indptr[r + 1];
-        d = b - a;
-        if (b < a) { bad = 1; d = 0; }
-        if (r == 0 && a != 0) bad = 1;
-        if (r == rows - 1 && (int64_t)b != nnz) bad = 1;
-        if (r > 0 && !bad) {
-            const int dp = a - indptr[r - 1];
-            if (d < dp) unsorted = 1;
-        }
+        int d = b - a;
+        bool row_bad = b < a;
+        if (row_bad) d = 0;
+        if (r == 0 && a != 0) row_bad = true;
+        if (r == rows - 1 && (int64_t)b != nnz) row_bad = true;
+        if (r > 0 && !row_bad && d < a - indptr[r - 1]) unsorted = 1;
+        bad |= row_bad;
         deg[r] = (uint32_t)d;
-        zero = d == 0;
-        if (d > kDegBound) { lrow = 1; lblk = (d + kDegBound - 1) / kDegBound; }
+        dmax = max(dmax, d);
+        zero += d == 0;
+        if (d > kDegBound) { lrow++; lblk += (d + kDegBound - 1) / kDegBound; }
     }
-    // wave-level combine, one atomic per wave and field
-    const unsigned long long any_bad = __ballot(bad), any_uns = __ballot(unsorted);
-    int m = d;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
-        m = max(m, __shfl_xor(m, off));
+        bad |= __shfl_xor(bad, off);
+        unsorted |= __shfl_xor(unsorted, off);
+        dmax = max(dmax, __shfl_xor(dmax, off));
+        zero += __shfl_xor(zero, off);
+        lrow += __shfl_xor(lrow, off);
         lblk += __shfl_xor(lblk, off);
     }
-    const int nz = __popcll(__ballot(zero)), nl = __popcll(__ballot(lrow));
+    const int w = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) {
-        if (any_bad) atomicOr(&st->bad_indptr, 1);
-        if (any_uns) atomicOr(&st->unsorted, 1);
-        if (m > 0) atomicMax(&st->max_degree, m);
-        if (nz) atomicAdd(&st->n_zero_rows, nz);
-        if (nl) atomicAdd(&st->n_long_rows, nl);
+        part[w][0] = bad; part[w][1] = unsorted; part[w][2] = dmax;
+        part[w][3] = zero; part[w][4] = lrow; part[w][5] = lblk;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int q = 1; q < kThreads / 64; q++) {
+            bad |= part[q][0]; unsorted |= part[q][1]; dmax = max(dmax, part[q][2]);
+            zero += part[q][3]; lrow += part[q][4]; lblk += part[q][5];
+        }
+        if (bad) atomicOr(&st->bad_indptr, 1);
+        if (unsorted) atomicOr(&st->unsorted, 1);
+        if (dmax > 0) atomicMax(&st->max_degree, dmax);
+        if (zero) atomicAdd(&st->n_zero_rows, zero);
+        if (lrow) atomicAdd(&st->n_long_rows, lrow);
         if (lblk) atomicAdd(&st->n_long_blocks, lblk);
     }
 }
@@ -482,7 +494,7 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
     if ((rc = deg.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
     if ((rc = st.alloc(sizeof(Stats)))) return rc;
     ACCEL_HIP(hipMemsetAsync(st.p, 0, sizeof(Stats), s));
-    degree_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(indptr_dev, rows, nnz,
+    degree_kernel<<<dim3(std::min(grid_for(rows), 2048u)), dim3(kThreads), 0, s>>>(indptr_dev, rows, nnz,
                                                                  deg.as<uint32_t>(), st.as<Stats>());
     Stats hs;
     ACCEL_HIP(hipMemcpyAsync(&hs, st.p, sizeof(Stats), hipMemcpyDeviceToHost, s));
@@ -592,7 +604,7 @@ int preprocess_device(accel_handle *h)
     if ((rc = deg.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
     if ((rc = st.alloc(sizeof(Stats)))) return rc;
     ACCEL_HIP(hipMemsetAsync(st.p, 0, sizeof(Stats), s));
-    degree_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(h->indptr, rows, nnz,
+    degree_kernel<<<dim3(std::min(grid_for(rows), 2048u)), dim3(kThreads), 0, s>>>(h->indptr, rows, nnz,
                                                                  deg.as<uint32_t>(), st.as<Stats>());
     Stats hs;
     ACCEL_HIP(hipMemcpyAsync(&hs, st.p, sizeof(Stats), hipMemcpyDeviceToHost, s));

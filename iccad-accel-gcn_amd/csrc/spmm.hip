@@ -56,9 +56,21 @@ __device__ __forceinline__ T stream_load(const T *p)
 #endif
 }
 
+#ifndef ACCEL_NT_GATHER
+#define ACCEL_NT_GATHER 0                 // experiment: gathers of X with the non-temporal hint
+#endif
+
 template <int VEC>
 __device__ __forceinline__ void load_vec(const float *__restrict__ p, float (&v)[VEC])
 {
+#if ACCEL_NT_GATHER
+    if constexpr (VEC == 4) {
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        const f4 t = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(p));
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        return;
+    }
+#endif
     if constexpr (VEC == 4) {
         const float4 t = *reinterpret_cast<const float4 *>(p);
         v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;

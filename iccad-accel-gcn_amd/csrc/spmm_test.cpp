@@ -1,0 +1,190 @@
+// spmm_test: command-line harness for the SPMM_ACCEL operator, the counterpart of
+// upstream's main.cu for the accel operator only.
+//
+//   spmm_test <graph> <dim>      check against a host CSR loop, then time (main.cu:186-194)
+//   spmm_test                    time every <graphs>/*.config for dim 16..128 (main.cu:195-219)
+//   options: --graphs DIR (default ../graphs/)  --meta DIR (default ../block_level_meta/)
+//
+// Input files, as upstream reads them (main.cu:62-63, data.h:7-21): <graph>.new_indptr and
+// <graph>.new_indices, raw little-endian int32.  Values are all 1 and vin ~ U[0,1) from
+// std::default_random_engine seeded with 123 (main.cu:90-93,114-121, value mode 3).
+// Output lines follow main.cu:40-49 and :161-167:
+//   err sum = <x>  validation pass!|fail!
+//   <i>/<n> <graph> <dim> accel <microseconds>
+// The check is upstream's: mean |out - ref| < 1e-3 (main.cu:18-51), with the reference
+// product computed here by a plain host loop where upstream calls cuSPARSE (main.cu:143-155).
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <filesystem>
+#include <iostream>
+#include <random>
+#include <vector>
+
+#include "accel_gcn.h"
+#include "spmm_accel.h"
+
+namespace {
+
+std::string base_dir = "../graphs/";
+std::string meta_dir = "../block_level_meta/";
+int dim_min = 16, dim_max = 128, interval = 1;
+int total_file_cnt = 0, current_file_cnt = 0;
+
+template <class T>
+bool read_managed(const std::string &path, T **arr, int64_t *count)
+{
+    int64_t n = 0;
+    if (accel_file_count(path.c_str(), &n) != ACCEL_OK) {
+        std::cerr << accel_last_error() << std::endl;
+        return false;
+    }
+    if (hipMallocManaged(reinterpret_cast<void **>(arr), (size_t)std::max<int64_t>(n, 1) * sizeof(T)) != hipSuccess) {
+        std::cerr << "hipMallocManaged failed for " << path << std::endl;
+        return false;
+    }
+    if (accel_file_read(path.c_str(), *arr, n) != ACCEL_OK) {
+        std::cerr << accel_last_error() << std::endl;
+        return false;
+    }
+    *count = n;
+    return true;
+}
+
+// the role cuSPARSE plays upstream: an independent product to check against
+void host_reference(const int *ptr, const int *idx, const float *val, const float *vin, float *out,
+                    int v_num, int dim)
+{
+    for (int r = 0; r < v_num; r++) {
+        float *y = out + (size_t)r * dim;
+        std::fill(y, y + dim, 0.0f);
+        for (int p = ptr[r]; p < ptr[r + 1]; p++) {
+            const float a = val[p];
+            const float *x = vin + (size_t)idx[p] * dim;
+            for (int j = 0; j < dim; j++) y[j] += a * x[j];
+        }
+    }
+}
+
+double check_err(const float *out, const float *ref, size_t len, bool &has_err)
+{
+    double err_sum = 0;
+    has_err = false;
+    for (size_t i = 0; i < len; i++) {
+        const double err = std::fabs((double)out[i] - (double)ref[i]);
+        err_sum += err;
+        if (err > 0.1 && !has_err) {
+            has_err = true;
+            std::cout << "err at " << i << std::endl;
+        }
+    }
+    std::cout << "err sum = " << err_sum << "  ";
+    std::cout << (err_sum / (double)len < 0.001 ? "validation pass!" : "validation fail!") << std::endl;
+    return err_sum;
+}
+
+int test_graph(const std::string &graph, int spec_dim, bool checking, bool timing)
+{
+    int lo = dim_min, hi = dim_max;
+    if (spec_dim > 0) lo = hi = spec_dim;
+
+    int *indptr = nullptr, *indices = nullptr;
+    int64_t n_ptr = 0, n_idx = 0;
+    if (!read_managed(base_dir + graph + ".new_indptr", &indptr, &n_ptr)) return 1;
+    if (!read_managed(base_dir + graph + ".new_indices", &indices, &n_idx)) return 1;
+    const int v_num = (int)n_ptr - 1, e_num = (int)n_idx;
+
+    float *val = nullptr, *vin = nullptr, *vout = nullptr;
+    const size_t dense = (size_t)v_num * hi;
+    if (hipMallocManaged(reinterpret_cast<void **>(&val), std::max<size_t>(e_num, 1) * sizeof(float)) != hipSuccess ||
+        hipMallocManaged(reinterpret_cast<void **>(&vin), std::max<size_t>(dense, 1) * sizeof(float)) != hipSuccess ||
+        hipMallocManaged(reinterpret_cast<void **>(&vout), std::max<size_t>(dense, 1) * sizeof(float)) != hipSuccess) {
+        std::cerr << "hipMallocManaged failed" << std::endl;
+        return 1;
+    }
+    std::default_random_engine engine;
+    engine.seed(123);
+    std::uniform_real_distribution<float> rd(0, 1);
+    std::fill(val, val + e_num, 1.0f);
+    std::generate(vin, vin + dense, [&]() { return rd(engine); });
+
+    SPMM_ACCEL accel(graph, indptr, indices, val, vin, vout, v_num, e_num, hi);
+    accel.set_meta_dir(meta_dir);
+    int rc = 0;
+    std::vector<float> ref;
+    for (int dim = lo; dim <= hi && rc == 0; dim += interval) {
+        if (checking) {
+            std::cout << "CHECKING ..." << std::endl;
+            if (accel.do_test(false, dim) < 0) {
+                std::cerr << "accel: " << accel.error() << std::endl;
+                rc = 1;
+                break;
+            }
+            ref.resize((size_t)v_num * dim);
+            host_reference(indptr, indices, val, vin, ref.data(), v_num, dim);
+            bool has_err = false;
+            std::cout << "checking accel" << std::endl;
+            const double e = check_err(vout, ref.data(), ref.size(), has_err);
+            if (!(e / (double)std::max<size_t>(ref.size(), 1) < 0.001)) rc = 2;
+        }
+        if (timing) {
+            std::cout << "TIMING ..." << std::endl;
+            const double t = accel.do_test(true, dim);
+            if (t < 0) {
+                std::cerr << "accel: " << accel.error() << std::endl;
+                rc = 1;
+                break;
+            }
+            std::cout << current_file_cnt << "/" << total_file_cnt << " " << graph << " " << dim
+                      << " accel " << t * 1e6 << std::endl;
+        }
+    }
+    (void)hipFree(indptr);
+    (void)hipFree(indices);
+    (void)hipFree(val);
+    (void)hipFree(vin);
+    (void)hipFree(vout);
+    return rc;
+}
+
+}  // namespace
+
+int main(int argc, char *argv[])
+{
+    std::vector<std::string> pos;
+    for (int i = 1; i < argc; i++) {
+        const std::string a = argv[i];
+        if (a == "--graphs" && i + 1 < argc) base_dir = argv[++i];
+        else if (a == "--meta" && i + 1 < argc) meta_dir = argv[++i];
+        else pos.push_back(a);
+    }
+    if (!base_dir.empty() && base_dir.back() != '/') base_dir += '/';
+    if (!meta_dir.empty() && meta_dir.back() != '/') meta_dir += '/';
+    int n_dev = 0;
+    if (accel_device_count(&n_dev) != ACCEL_OK || n_dev < 1) {
+        std::cerr << "spmm_test: no GPU (" << accel_last_error() << ")" << std::endl;
+        return 3;
+    }
+    if (pos.size() >= 2) {
+        std::cout << "dir = " << base_dir << std::endl;
+        return test_graph(pos[0], std::atoi(pos[1].c_str()), true, true);
+    }
+    namespace fs = std::filesystem;
+    std::error_code ec;
+    std::vector<std::string> graphs;
+    for (const auto &f : fs::directory_iterator(base_dir, ec))
+        if (f.path().extension() == ".config") graphs.push_back(f.path().stem().string());
+    if (ec) {
+        std::cerr << "spmm_test: cannot list " << base_dir << std::endl;
+        return 1;
+    }
+    std::sort(graphs.begin(), graphs.end());
+    total_file_cnt = (int)graphs.size();
+    int rc = 0;
+    for (const auto &g : graphs) {
+        current_file_cnt++;
+        rc |= test_graph(g, 0, false, true);
+        (void)hipDeviceSynchronize();
+    }
+    return rc;
+}

@@ -1,0 +1,77 @@
+"""bin/spmm_test, the C++ harness over SPMM_ACCEL (counterpart of main.cu)."""
+import re
+import subprocess
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import helpers
+from oracle import partition_oracle as po
+
+ROOT = Path(__file__).resolve().parent.parent
+EXE = ROOT / "iccad-accel-gcn_amd" / "bin" / "spmm_test"
+
+
+def write_graph(tmp, name, seed, n_long=3):
+    """<name>.config/.new_indptr/.new_indices in upstream's layout (degree-sorted
+    rows, raw int32), plus the matching <name>.block4."""
+    g0 = helpers.graph_from_degrees(helpers.degree_mix(seed=seed, n_long=n_long), seed=seed)
+    n = g0.n_rows
+    # square adjacency, as upstream assumes (vin has v_num rows)
+    g0.indices[:] = g0.indices % n
+    perm = po.degree_sort(g0.indptr)
+    sip, six, _ = po.permute_csr(g0.indptr, g0.indices, g0.values, perm)
+    graphs, meta = tmp / "graphs", tmp / "block_level_meta"
+    graphs.mkdir(exist_ok=True)
+    meta.mkdir(exist_ok=True)
+    (graphs / f"{name}.config").write_text("")
+    sip.astype("<i4").tofile(graphs / f"{name}.new_indptr")
+    six.astype("<i4").tofile(graphs / f"{name}.new_indices")
+    po.partition_closed_form(sip).astype("<i4").tofile(meta / f"{name}.block4")
+    return graphs, meta
+
+
+def test_cli_without_gpu_says_so(pkg):
+    if pkg.device_count() > 0:
+        pytest.skip("a GPU is present")
+    assert EXE.exists(), "spmm_test was not built"
+    r = subprocess.run([str(EXE), "g", "16"], capture_output=True, text=True)
+    assert r.returncode == 3 and "no GPU" in r.stderr
+
+
+@pytest.mark.gpu
+def test_cli_check_and_timing(gpu, tmp_path):
+    graphs, meta = write_graph(tmp_path, "mix", seed=11)
+    r = subprocess.run([str(EXE), "--graphs", str(graphs), "--meta", str(meta), "mix", "60"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "validation pass!" in r.stdout
+    m = re.search(r"^0/0 mix 60 accel ([0-9.eE+-]+)$", r.stdout, re.M)    # main.cu:161-167 line format
+    assert m and 0 < float(m.group(1)) < 1e6
+
+
+@pytest.mark.gpu
+def test_cli_refuses_stale_metadata(gpu, tmp_path):
+    graphs, meta = write_graph(tmp_path, "mix", seed=12)
+    b = np.fromfile(meta / "mix.block4", dtype="<i4")
+    b[2] += 1
+    b.tofile(meta / "mix.block4")
+    r = subprocess.run([str(EXE), "--graphs", str(graphs), "--meta", str(meta), "mix", "32"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "metadata differs" in r.stderr
+
+
+@pytest.mark.gpu
+def test_cli_sweep_mode(gpu, tmp_path):
+    for i, name in enumerate(("a", "b")):
+        graphs, meta = write_graph(tmp_path, name, seed=20 + i, n_long=1)
+    # sweep = every *.config, dims 16..128 (main.cu:12,195-219); without a metadata
+    # directory the operator builds everything itself
+    r = subprocess.run([str(EXE), "--graphs", str(graphs), "--meta", str(tmp_path / "none")],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    lines = re.findall(r"^(\d)/2 (\w) (\d+) accel ([0-9.eE+-]+)$", r.stdout, re.M)
+    assert len(lines) == 2 * 113
+    assert {(l[0], l[1]) for l in lines} == {("1", "a"), ("2", "b")}
+    assert [int(l[2]) for l in lines[:113]] == list(range(16, 129))
