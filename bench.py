@@ -66,12 +66,41 @@ def cpu_baseline(g, X, N, budget_s=15.0):
                       f"({nz} of {g.nnz} non-zeros), N={N}, 1 thread"}, n_rows, Y
 
 
+def fixture_graph(pkg, name, seed=0):
+    """A graph with exactly the degree sequence of one of the reference's
+    benchmark graphs (recovered from its golden .block4 metadata: degree, first
+    row and row count of every block; rows no block covers have degree 0), rows
+    in shuffled order, columns uniform random (distinct inside a row), values
+    GCN-normalised.  The real edge lists are not available offline."""
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "golden"))
+    import block4_codec
+    b = block4_codec.load(name).astype(np.int64)
+    is_long = b[:, 0] > 384
+    first = np.ones(len(b), dtype=bool)
+    first[1:] = ~(is_long[1:] & (b[1:, 1] == b[:-1, 1]))
+    b = b[first]
+    n_rows_blk = np.where(b[:, 0] > 384, 1, b[:, 3] & 0xFFFF)
+    n = int((b[:, 1] + n_rows_blk).max())
+    deg = np.zeros(n, dtype=np.int64)
+    deg[np.repeat(b[:, 1], n_rows_blk) + (np.arange(n_rows_blk.sum()) - np.repeat(np.cumsum(n_rows_blk) - n_rows_blk, n_rows_blk))] = np.repeat(b[:, 0], n_rows_blk)
+    rng = np.random.default_rng(seed)
+    deg = rng.permutation(deg)
+    src = np.repeat(np.arange(n, dtype=np.int64), deg)
+    dst = rng.integers(0, n, size=src.size, dtype=np.int64)
+    syn = pkg.synthetic
+    indptr, indices = syn._csr_from_edges(src, dst, n, n)
+    g = syn.Graph(name, indptr, indices, syn._gcn_values(indptr, indices), n, n)
+    return g
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=4)
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--workload", default="cfg4",
+                    help="cfg1..cfg5, or fixture:<name> for the degree sequence of one of the "
+                         "reference's graphs (e.g. fixture:OVCAR-8H, fixture:ppa)")
     ap.add_argument("--N", type=int, default=0, help="columns of X (default: the workload's first)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the scipy baseline and the check")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
@@ -98,10 +127,15 @@ def main():
                           "bytes_read_per_launch": words * 4, "bytes_written_per_launch": words * 4}))
         return
     syn = pkg.synthetic
-    N = a.N or syn.WORKLOAD_N[a.workload][0]
+    N = a.N or syn.WORKLOAD_N.get(a.workload, (64,))[0]
 
     t0 = time.time()
-    g = syn.WORKLOADS[a.workload]()
+    if a.workload.startswith("fixture:"):
+        g = fixture_graph(pkg, a.workload.split(":", 1)[1])
+    elif a.workload in syn.WORKLOADS:
+        g = syn.WORKLOADS[a.workload]()
+    else:
+        sys.exit(f"bench.py: unknown workload {a.workload}")
     X = syn.dense_operand(a.workload, g.n_cols, N)
     log(f"[bench] {a.workload}: rows={g.n_rows} nnz={g.nnz} N={N} generated in {time.time() - t0:.1f}s")
 

@@ -68,6 +68,7 @@ SIGNATURES = {
     "accel_check_block4": (C.c_int, [vp, i32p, C.c_int64]),
     "accel_get_info": (C.c_int, [vp, C.POINTER(Info)]),
     "accel_get_block4": (C.c_int, [vp, i32p, C.c_int64]),
+    "accel_get_plan": (C.c_int, [vp, i32p, C.c_int64, i64p]),
     "accel_get_perm": (C.c_int, [vp, i32p, C.c_int64]),
     "accel_get_sorted_csr": (C.c_int, [vp, i32p, i32p, f32p]),
     "accel_run": (C.c_int, [vp, vp, vp, C.c_int32, vp]),

@@ -417,6 +417,18 @@ int accel_get_sorted_csr(const accel_handle *h, int32_t *indptr, int32_t *idx, f
     return ACCEL_OK;
 }
 
+int accel_get_plan(const accel_handle *h, int32_t *out, int64_t cap_units, int64_t *n_units)
+{
+    clear_error();
+    if (!h || !n_units || cap_units < 0) { set_error("accel_get_plan: bad argument"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_get_plan: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    *n_units = h->n_units;
+    const int64_t take = std::min(cap_units, h->n_units);
+    if (out && take > 0)
+        ACCEL_HIP(hipMemcpy(out, h->work, sizeof(int32_t) * 4 * (size_t)take, hipMemcpyDeviceToHost));
+    return ACCEL_OK;
+}
+
 int accel_check_block4(accel_handle *h, const int32_t *block4_host, int64_t n_blocks)
 {
     clear_error();

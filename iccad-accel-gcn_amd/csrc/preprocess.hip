@@ -429,6 +429,98 @@ __global__ __launch_bounds__(kThreads) void emit_block4_kernel(
     block4[at] = make_int4(d, (int)r, loc, (w << 16) + n);
 }
 
+// ---------------------------------------------------------------------------
+// Launch plan (work list), built on the GPU.  See build_work_list below.
+// ---------------------------------------------------------------------------
+struct PlanParams {
+    int queue_long[kXcds];   // long-row units already in each queue
+    int quota[kXcds];        // block4 entries of short rows each queue takes
+};
+
+__device__ __forceinline__ int64_t plan_index(int queue, int pos)
+{
+    // queue q, position p  ->  slot of wavefront (p % 4) in workgroup (p / 4) * 8 + q
+    return ((int64_t)(pos / kWavesPerGroup) * kXcds + queue) * kWavesPerGroup + pos % kWavesPerGroup;
+}
+
+__global__ __launch_bounds__(kThreads) void long_unit_count_kernel(
+    const int *__restrict__ gcount, int n_long, int *__restrict__ row_units,
+    int *__restrict__ grp_units)
+{
+    const int lr = blockIdx.x * kThreads + threadIdx.x;
+    if (lr >= n_long) return;
+    int tot = 0;
+#pragma unroll
+    for (int g = 0; g < kXcds; g++) {
+        const int u = (gcount[(int64_t)lr * kXcds + g] + kDegBound - 1) / kDegBound;
+        grp_units[(int64_t)g * n_long + (n_long - 1 - lr)] = u;   // largest rows first
+        tot += u;
+    }
+    row_units[lr] = tot;
+}
+
+__global__ void plan_totals_kernel(const int *__restrict__ grp_pos, int n_long, int *__restrict__ out)
+{
+    const int g = threadIdx.x;
+    if (g <= kXcds) out[g] = grp_pos[(int64_t)g * n_long];   // g == 8: grand total
+}
+
+__global__ __launch_bounds__(kThreads) void emit_long_units_kernel(
+    const int *__restrict__ gcount, const int32_t *__restrict__ s_indptr, int64_t first_long,
+    const int *__restrict__ slot, const int *__restrict__ grp_pos, int n_long,
+    int4 *__restrict__ work)
+{
+    const int t = blockIdx.x * kThreads + threadIdx.x;
+    if (t >= n_long * kXcds) return;
+    const int lr = t / kXcds, g = t % kXcds;
+    const int c = gcount[(int64_t)lr * kXcds + g];
+    if (c == 0) return;
+    int c_before = 0, u_before = 0;
+    for (int q = 0; q < g; q++) {
+        const int cq = gcount[(int64_t)lr * kXcds + q];
+        c_before += cq;
+        u_before += (cq + kDegBound - 1) / kDegBound;
+    }
+    const int row = (int)(first_long + lr);
+    const int loc = s_indptr[row] + c_before;
+    const int pos0 = grp_pos[(int64_t)g * n_long + (n_long - 1 - lr)] - grp_pos[(int64_t)g * n_long];
+    const int sl = slot[lr] + u_before;
+    for (int k = 0, off = 0; off < c; k++, off += kDegBound)
+        work[plan_index(g, pos0 + k)] =
+            make_int4(kDegBound + 1 + sl + k, row, loc + off, min(kDegBound, c - off));
+}
+
+__global__ __launch_bounds__(kThreads) void emit_short_units_kernel(
+    const int4 *__restrict__ block4, int n_short, PlanParams pp, int4 *__restrict__ work)
+{
+    const int i = blockIdx.x * kThreads + threadIdx.x;   // dealing order: highest degree first
+    if (i >= n_short) return;
+    // entries are dealt in rounds; in round t every queue with quota > t takes one,
+    // in queue order.  dealt(t) = sum_q min(quota_q, t) entries precede round t.
+    int lo = 0, hi = 0;
+#pragma unroll
+    for (int q = 0; q < kXcds; q++) hi = max(hi, pp.quota[q]);
+    while (lo < hi) {                                  // largest t with dealt(t) <= i
+        const int mid = (lo + hi + 1) >> 1;
+        int dealt = 0;
+#pragma unroll
+        for (int q = 0; q < kXcds; q++) dealt += min(pp.quota[q], mid);
+        if (dealt <= i) lo = mid; else hi = mid - 1;
+    }
+    int j = i;
+#pragma unroll
+    for (int q = 0; q < kXcds; q++) j -= min(pp.quota[q], lo);
+    int queue = 0;
+#pragma unroll
+    for (int q = kXcds - 1; q >= 0; q--) {
+        // the j-th queue (ascending) that is still open in round lo
+        int open_before = 0;
+        for (int r = 0; r < q; r++) open_before += pp.quota[r] > lo;
+        if (pp.quota[q] > lo && open_before == j) queue = q;
+    }
+    work[plan_index(queue, pp.queue_long[queue] + lo)] = block4[n_short - 1 - i];
+}
+
 struct DevBuf {  // frees on scope exit
     void *p = nullptr;
     ~DevBuf() { if (p) (void)hipFree(p); }
@@ -516,68 +608,90 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
 // Workgroups are dispatched to the eight dies round-robin (workgroup i runs on
 // die i % 8), so the list is laid out as eight interleaved queues: units of
 // column group g of the long rows go to queue g, whose die then keeps that
-// share of X in its own L2; block4 entries of short rows fill all queues
-// evenly.  Every queue runs its heaviest units first.
-static int build_work_list(accel_handle *h, const std::vector<int32_t> &long_ptr,
-                           const std::vector<int> &group_count, int64_t first_long, hipStream_t s)
+// share of X in its own L2; block4 entries of short rows are dealt to the
+// queues in rounds until all queues are equally long.  Every queue runs its
+// heaviest units first.  Only nine integers travel to the host (the queue
+// lengths), to size the list.
+static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_indptr,
+                           int64_t first_long, hipStream_t s)
 {
-    struct Unit { int32_t x, y, z, w; };
-    const int64_t n_long = (int64_t)long_ptr.size() - 1;
+    const int64_t n_long = h->n_long_rows;
     const int64_t n_short = h->n_blocks - h->n_long_blocks;
-    std::vector<Unit> short_units((size_t)n_short);
-    if (n_short > 0)
-        ACCEL_HIP(hipMemcpyAsync(short_units.data(), h->block4, sizeof(Unit) * (size_t)n_short,
-                                 hipMemcpyDeviceToHost, s));
-    // partial-sum slots: contiguous per long row, in row order
-    std::vector<int32_t> slot((size_t)n_long + 1, 0);
-    for (int64_t lr = 0; lr < n_long; lr++) {
-        int u = 0;
-        for (int g = 0; g < kXcds; g++) u += (group_count[(size_t)lr * kXcds + g] + kDegBound - 1) / kDegBound;
-        slot[(size_t)lr + 1] = slot[(size_t)lr] + u;
-    }
-    const int64_t n_long_units = slot[(size_t)n_long];
-    std::vector<Unit> queue[kXcds];
-    for (int64_t lr = n_long - 1; lr >= 0; lr--) {      // largest rows first
-        int32_t at = long_ptr[(size_t)lr], sl = slot[(size_t)lr];
-        for (int g = 0; g < kXcds; g++) {
-            const int c = group_count[(size_t)lr * kXcds + g];
-            for (int off = 0; off < c; off += kDegBound)
-                queue[g].push_back(Unit{kDegBound + 1 + sl++, (int32_t)(first_long + lr), at + off,
-                                        std::min(kDegBound, c - off)});
-            at += c;
-        }
-    }
-    ACCEL_HIP(hipStreamSynchronize(s));
-    size_t longest = 0;
-    for (auto &q : queue) longest = std::max(longest, q.size());
-    const size_t total = (size_t)n_long_units + (size_t)n_short;
-    size_t per_queue = std::max(longest, (total + kXcds - 1) / kXcds);
-    per_queue = (per_queue + kWavesPerGroup - 1) / kWavesPerGroup * kWavesPerGroup;
-    // short entries, highest degree first, dealt to the queues that still have room
-    {
-        int g = 0;
-        for (int64_t e = n_short - 1; e >= 0; e--) {
-            int tries = 0;
-            while (queue[g].size() >= per_queue && tries < kXcds) { g = (g + 1) % kXcds; tries++; }
-            queue[g].push_back(short_units[(size_t)e]);
-            g = (g + 1) % kXcds;
-        }
-    }
-    for (auto &q : queue) q.resize(per_queue, Unit{0, 0, 0, 0});
-    std::vector<Unit> work(per_queue * kXcds);
-    for (size_t q = 0; q < per_queue / kWavesPerGroup; q++)
-        for (int g = 0; g < kXcds; g++)
-            for (int w = 0; w < kWavesPerGroup; w++)
-                work[(q * kXcds + g) * kWavesPerGroup + w] = queue[g][q * kWavesPerGroup + w];
-    h->n_units = (int64_t)work.size();
-    h->n_long_units = n_long_units;
-    DevBuf dwork, dslot;
+    DevBuf row_units, grp_units, sums, totals, dslot;
     int rc;
-    if ((rc = dwork.alloc(sizeof(Unit) * work.size()))) return rc;
-    if ((rc = dslot.alloc(sizeof(int32_t) * slot.size()))) return rc;
-    if (!work.empty())
-        ACCEL_HIP(hipMemcpy(dwork.p, work.data(), sizeof(Unit) * work.size(), hipMemcpyHostToDevice));
-    ACCEL_HIP(hipMemcpy(dslot.p, slot.data(), sizeof(int32_t) * slot.size(), hipMemcpyHostToDevice));
+    int tot[kXcds + 1] = {0};
+    if ((rc = dslot.alloc(sizeof(int) * (size_t)(n_long + 1)))) return rc;
+    if (n_long > 0) {
+        if ((rc = row_units.alloc(sizeof(int) * (size_t)n_long))) return rc;
+        if ((rc = grp_units.alloc(sizeof(int) * (size_t)(n_long * kXcds + 1)))) return rc;
+        if ((rc = sums.alloc(sizeof(int) * (size_t)(n_long * kXcds / kTile + 4)))) return rc;
+        if ((rc = totals.alloc(sizeof(int) * (kXcds + 1)))) return rc;
+        long_unit_count_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(
+            gcount, (int)n_long, row_units.as<int>(), grp_units.as<int>());
+        if ((rc = device_scan<SumOp, false>(row_units.as<int>(), n_long, dslot.as<int>(),
+                                            dslot.as<int>() + n_long, sums.as<int>(), s)))
+            return rc;
+        if ((rc = device_scan<SumOp, false>(grp_units.as<int>(), n_long * kXcds, grp_units.as<int>(),
+                                            grp_units.as<int>() + n_long * kXcds, sums.as<int>(), s)))
+            return rc;
+        plan_totals_kernel<<<dim3(1), dim3(64), 0, s>>>(grp_units.as<int>(), (int)n_long,
+                                                      totals.as<int>());
+        ACCEL_HIP(hipMemcpyAsync(tot, totals.p, sizeof(tot), hipMemcpyDeviceToHost, s));
+        ACCEL_HIP(hipStreamSynchronize(s));
+    } else {
+        ACCEL_HIP(hipMemsetAsync(dslot.p, 0, sizeof(int), s));
+    }
+    PlanParams pp;
+    int64_t longest = 0;
+    for (int g = 0; g < kXcds; g++) {
+        pp.queue_long[g] = tot[g + 1] - tot[g];
+        longest = std::max<int64_t>(longest, pp.queue_long[g]);
+    }
+    const int64_t n_long_units = tot[kXcds];
+    const int64_t total = n_long_units + n_short;
+    int64_t per_queue = std::max(longest, (total + kXcds - 1) / kXcds);
+    per_queue = (per_queue + kWavesPerGroup - 1) / kWavesPerGroup * kWavesPerGroup;
+    // quotas: fill the queues level, shortest first, until the short entries are used up
+    {
+        int64_t left = n_short;
+        for (int g = 0; g < kXcds; g++) pp.quota[g] = 0;
+        // raise a common fill level: queue g takes max(0, level - queue_long[g])
+        int64_t lo = 0, hi = per_queue;
+        auto taken = [&](int64_t level) {
+            int64_t t = 0;
+            for (int g = 0; g < kXcds; g++) t += std::max<int64_t>(0, level - pp.queue_long[g]);
+            return t;
+        };
+        while (lo < hi) {                              // largest level with taken(level) <= n_short
+            const int64_t mid = (lo + hi + 1) / 2;
+            if (taken(mid) <= n_short) lo = mid; else hi = mid - 1;
+        }
+        for (int g = 0; g < kXcds; g++) {
+            pp.quota[g] = (int)std::max<int64_t>(0, lo - pp.queue_long[g]);
+            left -= pp.quota[g];
+        }
+        for (int g = 0; g < kXcds && left > 0; g++)    // remainder: one more for the first queues with room
+            if (pp.queue_long[g] + pp.quota[g] < per_queue) { pp.quota[g]++; left--; }
+        if (left != 0) {
+            set_error("internal: launch plan could not place %lld block4 entries", (long long)left);
+            return ACCEL_ERR_ARG;
+        }
+    }
+    const int64_t n_units = per_queue * kXcds;
+    DevBuf dwork;
+    if ((rc = dwork.alloc(sizeof(int4) * (size_t)n_units))) return rc;
+    if (n_units > 0 && (rc = fill_u32(dwork.p, 0u, (size_t)n_units * 4, s))) return rc;
+    if (n_long > 0)
+        emit_long_units_kernel<<<dim3(grid_for(n_long * kXcds)), dim3(kThreads), 0, s>>>(
+            gcount, s_indptr, first_long, dslot.as<int>(), grp_units.as<int>(), (int)n_long,
+            dwork.as<int4>());
+    if (n_short > 0)
+        emit_short_units_kernel<<<dim3(grid_for(n_short)), dim3(kThreads), 0, s>>>(
+            reinterpret_cast<const int4 *>(h->block4), (int)n_short, pp, dwork.as<int4>());
+    ACCEL_HIP(hipGetLastError());
+    ACCEL_HIP(hipStreamSynchronize(s));
+    h->n_units = n_units;
+    h->n_long_units = n_long_units;
     h->work = static_cast<int32_t *>(dwork.release());
     h->long_slot = static_cast<int32_t *>(dslot.release());
     return ACCEL_OK;
@@ -674,14 +788,13 @@ int preprocess_device(accel_handle *h)
     // column group.  The caller's arrays are used in place only when the input
     // was already sorted and has no long row.
     const int64_t n_long = hs.n_long_rows, first_long = rows - n_long;
-    std::vector<int32_t> long_ptr((size_t)n_long + 1);   // s_indptr[first_long .. rows]
-    ACCEL_HIP(hipMemcpyAsync(long_ptr.data(), sip.as<int32_t>() + first_long,
-                             sizeof(int32_t) * long_ptr.size(), hipMemcpyDeviceToHost, s));
+    int32_t nnz_short32 = 0;                             // non-zeros of the rows with degree <= 384
+    ACCEL_HIP(hipMemcpyAsync(&nnz_short32, sip.as<int32_t>() + first_long, sizeof(int32_t),
+                             hipMemcpyDeviceToHost, s));
     ACCEL_HIP(hipStreamSynchronize(s));
-    const int64_t nnz_short = long_ptr[0];
+    const int64_t nnz_short = nnz_short32;
     const bool own_copy = !h->identity_perm || n_long > 0;
     DevBuf sidx, sval, permbuf, gcount;
-    std::vector<int> group_count((size_t)n_long * kXcds);
     if (own_copy) {
         if ((rc = sidx.alloc(sizeof(int32_t) * (size_t)nnz))) return rc;
         if ((rc = sval.alloc(sizeof(float) * (size_t)nnz))) return rc;
@@ -703,12 +816,10 @@ int preprocess_device(accel_handle *h)
                                      hipMemcpyDeviceToDevice, s));
         }
         if (n_long > 0) {
-            if ((rc = gcount.alloc(sizeof(int) * group_count.size()))) return rc;
+            if ((rc = gcount.alloc(sizeof(int) * (size_t)n_long * kXcds))) return rc;
             group_long_rows_kernel<<<dim3((unsigned)n_long), dim3(kThreads), 0, s>>>(
                 h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), first_long, sidx.as<int32_t>(),
                 sval.as<float>(), gcount.as<int>());
-            ACCEL_HIP(hipMemcpyAsync(group_count.data(), gcount.p, sizeof(int) * group_count.size(),
-                                     hipMemcpyDeviceToHost, s));
         }
         ACCEL_HIP(hipGetLastError());
     }
@@ -722,7 +833,7 @@ int preprocess_device(accel_handle *h)
     h->n_blocks = nb;
 
     // ---- work list ------------------------------------------------------------
-    if ((rc = build_work_list(h, long_ptr, group_count, first_long, s))) return rc;
+    if ((rc = build_work_list(h, gcount.as<int>(), sip.as<int32_t>(), first_long, s))) return rc;
 
     h->s_indptr = static_cast<int32_t *>(sip.release());
     if (!own_copy) {

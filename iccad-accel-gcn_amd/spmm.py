@@ -77,6 +77,15 @@ class AccelSpMM:
         check(lib().accel_get_block4(self._h, ptr(out, C.c_int32), out.shape[0]))
         return out
 
+    def plan(self) -> np.ndarray:
+        """The launch plan: one (x, y, z, w) row per wavefront (see accel_get_plan)."""
+        self.info
+        n = C.c_int64(0)
+        check(lib().accel_get_plan(self._h, None, 0, C.byref(n)))
+        out = np.empty((n.value, 4), dtype=np.int32)
+        check(lib().accel_get_plan(self._h, ptr(out, C.c_int32), n.value, C.byref(n)))
+        return out
+
     def perm(self) -> np.ndarray:
         self.info
         out = np.empty(self.n_rows, dtype=np.int32)

@@ -128,6 +128,16 @@ int accel_get_block4(const accel_handle *h, int32_t *out, int64_t cap_blocks);
 int accel_get_perm(const accel_handle *h, int32_t *out, int64_t cap_rows);
 int accel_get_sorted_csr(const accel_handle *h, int32_t *indptr, int32_t *idx, float *val);
 
+/* The launch plan derived from block4 (no counterpart upstream, where the grid
+ * is simply one thread block per block4 entry, spmm_accel.cu:128): one int4
+ * (x, y, z, w) per wavefront, four per workgroup.  x <= 384: a block4 entry of
+ * whole rows, verbatim.  x > 384: a piece of a long row: partial-sum slot
+ * x - 385, sorted row y, first non-zero z, length w <= 384.  w == 0: padding.
+ * Workgroup i runs on die i % 8, so units 4*i .. 4*i+3 belong to queue i % 8;
+ * the pieces of long rows in queue g only hold columns c with (c >> 3) & 7 == g.
+ * Writes up to cap_units quadruples to out (may be NULL) and the count to *n_units. */
+int accel_get_plan(const accel_handle *h, int32_t *out, int64_t cap_units, int64_t *n_units);
+
 /* run: replaces SPMM_ACCEL::run (spmm_accel.cu:104-108).  Y = A X with beta = 0:
  * every row of Y is written exactly once, rows of degree 0 receive zeros (the
  * upstream kernel leaves them untouched and accumulates into the rest,

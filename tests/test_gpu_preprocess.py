@@ -170,3 +170,54 @@ def test_call_order_and_arguments(gpu):
     assert e.value.status == gpu._lib.ERR_ARG
     buf.close()
     op.close()
+
+
+def check_plan(op, n_cols):
+    """The launch plan covers every non-zero exactly once, keeps block4 entries of
+    short rows verbatim, and queues each piece of a long row on the die that owns
+    its column group."""
+    plan = op.plan().astype(np.int64)
+    b4 = op.block4().astype(np.int64)
+    sip, six, _ = op.sorted_csr()
+    assert plan.shape[0] % 32 == 0                       # 8 queues x 4 wavefronts
+    live = plan[plan[:, 3] != 0]
+    short = live[live[:, 0] <= 384]
+    long_ = live[live[:, 0] > 384]
+    b4_short = b4[b4[:, 0] <= 384]
+    assert sorted(map(tuple, short)) == sorted(map(tuple, b4_short))
+    covered = np.zeros(six.size, dtype=np.int32)
+    for x, y, z, w in long_:
+        covered[z:z + w] += 1
+        assert 0 < w <= 384 and sip[y] <= z and z + w <= sip[y + 1]
+    for d, r, loc, info in short:
+        covered[loc:loc + d * (info & 0xFFFF)] += 1
+    assert np.all(covered == 1)
+    # queue of unit e is (e // 4) % 8
+    queue = (np.arange(plan.shape[0]) // 4) % 8
+    for e in np.flatnonzero((plan[:, 3] != 0) & (plan[:, 0] > 384)):
+        x, y, z, w = plan[e]
+        assert np.all(po.column_group(six[z:z + w]) == queue[e])
+    # partial-sum slots: 0 .. n-1, each once, contiguous per row in row order
+    slots = long_[:, 0] - 385
+    assert sorted(slots.tolist()) == list(range(len(long_)))
+    order = np.argsort(slots)
+    assert np.all(np.diff(long_[order, 1]) >= 0)
+    # queues are balanced to within one workgroup
+    per_queue = [int((plan[queue == q][:, 3] != 0).sum()) for q in range(8)]
+    if len(long_) == 0:
+        assert max(per_queue) - min(per_queue) <= 1
+
+
+@pytest.mark.parametrize("seed,n_long", [(0, 0), (1, 3), (2, 9)])
+def test_launch_plan(gpu, seed, n_long):
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=seed, n_long=n_long), seed=seed)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    check_plan(op, g.n_cols)
+    op.close()
+
+
+def test_launch_plan_hub_graph(gpu):
+    g = gpu.synthetic.hub_graph_small()
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    check_plan(op, g.n_cols)
+    op.close()
