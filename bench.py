@@ -93,6 +93,33 @@ def fixture_graph(pkg, name, seed=0):
     return g
 
 
+def rocsparse_baseline(pkg, op, g, dX, N, iters=10):
+    """Vendor-library CSR SpMM on the same resident operands (comparison only, as
+    upstream compares with cuSPARSE; never part of `value`)."""
+    import ctypes as C
+    path = os.path.join(os.path.dirname(str(pkg._lib.LIB_PATH)), "libaccelgcn_baselines.so")
+    L = C.CDLL(path)
+    L.baseline_last_error.restype = C.c_char_p
+    bufs = [pkg.DeviceBuffer.from_numpy(a) for a in (g.indptr, g.indices, g.values)]
+    dY = pkg.DeviceBuffer(g.n_rows * N * 4)
+    out = {}
+    for name, alg in (("default", 0), ("row_split", 4), ("nnz_split", 5), ("merge_path", 9)):
+        ms = (C.c_float * iters)()
+        pre = C.c_float(0)
+        rc = L.baseline_rocsparse_spmm(C.c_void_p(bufs[0].address), C.c_void_p(bufs[1].address),
+                                       C.c_void_p(bufs[2].address), C.c_int64(g.n_rows), C.c_int64(g.n_cols),
+                                       C.c_int64(g.nnz), C.c_void_p(dX.address), C.c_void_p(dY.address),
+                                       C.c_int32(N), alg, 3, iters, ms, C.byref(pre))
+        if rc != 0:
+            out[name] = {"error": L.baseline_last_error().decode()}
+            continue
+        out[name] = {"ms": round(float(np.median(list(ms))), 5), "preprocess_ms": round(pre.value, 3)}
+    Yr = dY.to_numpy(np.float32, (g.n_rows, N))
+    for b in bufs + [dY]:
+        b.close()
+    return out, Yr
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -103,6 +130,8 @@ def main():
                          "reference's graphs (e.g. fixture:OVCAR-8H, fixture:ppa)")
     ap.add_argument("--N", type=int, default=0, help="columns of X (default: the workload's first)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the scipy baseline and the check")
+    ap.add_argument("--compare-rocsparse", action="store_true",
+                    help="also time rocSPARSE's CSR SpMM on the same operands (comparison only)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run the plain copy kernel over this many MiB, --steps times "
                          "(known-size reference for the FETCH_SIZE / WRITE_SIZE counters)")
@@ -185,6 +214,13 @@ def main():
                      "algorithmic_bytes": alg_bytes},
     }
 
+    if a.compare_rocsparse:
+        rs, Yr = rocsparse_baseline(pkg, op, g, dX, N)
+        Ymine = dY.to_numpy(np.float32, (g.n_rows, N))
+        best = min((v["ms"] for v in rs.values() if "ms" in v), default=None)
+        result["rocsparse"] = {"algorithms": rs, "best_ms": best,
+                               "speedup_vs_best": round(best / float(np.mean(tot_ms)), 3) if best else None,
+                               "max_abs_diff_vs_last_alg": float(np.max(np.abs(Ymine - Yr))) if Yr.size else 0.0}
     if not a.no_cpu:
         base, n_rows, Yc = cpu_baseline(g, X, N)
         result["cpu_baseline"] = base

@@ -44,6 +44,9 @@ constexpr int kZeroFloats = 16384;        // floats zero-filled per extra workgr
 #ifndef ACCEL_NT_STORE
 #define ACCEL_NT_STORE 0                  // 1: Y rows are stored with the non-temporal hint
 #endif
+#ifndef ACCEL_PREDICATED
+#define ACCEL_PREDICATED 1                // 1: one masked batch loop; 0: full batches + scalar tail
+#endif
 constexpr int kUnroll = ACCEL_UNROLL;
 
 template <class T>
@@ -145,6 +148,10 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     const int d = is_long ? info : deg;                 // spmm_accel.cu:28: non-zeros per row here
     const int total_nz = n_rows * d;
 
+    // output row of each of the unit's rows, fetched up front (lane r holds row r)
+    int my_out = row0 + lane;
+    if (!is_long && perm && lane < n_rows) my_out = perm[row0 + lane];
+
     // stage the entry's (column, value) pairs: all loads are issued before the first LDS write
     int2 *st = stage[wv];
     {
@@ -196,6 +203,33 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
             if (live) {
                 const int2 *row_st = st + r * d;
                 const float *xcol = X + col;
+#if ACCEL_PREDICATED
+                // every batch issues up to kUnroll gathers; lanes past the end of the
+                // row are masked, so a row costs ceil(d / (gp * kUnroll)) round trips
+                for (int o = k; o < d; o += kUnroll * gp) {
+                    int2 p[kUnroll];
+                    float x[kUnroll][VEC];
+                    bool ok[kUnroll];
+#pragma unroll
+                    for (int u = 0; u < kUnroll; u++) {
+                        const int ou = o + u * gp;
+                        ok[u] = ou < d;
+                        p[u] = row_st[ok[u] ? ou : k];
+                    }
+#pragma unroll
+                    for (int u = 0; u < kUnroll; u++) {
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) x[u][v] = 0.0f;
+                        if (ok[u]) load_vec<VEC>(xcol + (int64_t)p[u].x * N, x[u]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < kUnroll; u++) {
+                        const float a = ok[u] ? __int_as_float(p[u].y) : 0.0f;
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[u][v], acc[v]);
+                    }
+                }
+#else
                 int o = k;
                 for (; o + (kUnroll - 1) * gp < d; o += kUnroll * gp) {
                     int2 p[kUnroll];
@@ -219,19 +253,19 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 #pragma unroll
                     for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[v], acc[v]);
                 }
+#endif
             }
             // add the gp partial sums of each row (all lanes take part)
             for (int m = L; m < (L << lg); m <<= 1) {
 #pragma unroll
                 for (int v = 0; v < VEC; v++) acc[v] += __shfl_xor(acc[v], m);
             }
+            const int64_t out_row = __shfl(my_out, r < n_rows ? r : 0);
             if (live && k == 0) {
-                if (is_long) {
+                if (is_long)
                     store_vec<VEC>(partial + (int64_t)(deg - (kDegBound + 1)) * N + col, acc);
-                } else {
-                    const int64_t out_row = perm ? perm[row0 + r] : row0 + r;
+                else
                     store_out<VEC>(Y + out_row * N + col, acc);
-                }
             }
         }
     }

@@ -1,0 +1,85 @@
+"""accel_run on caller-owned HIP streams and inside a captured HIP graph: the run
+path launches kernels only (no synchronisation, no allocation once the scratch
+buffer for that N exists), so it can be replayed from a graph."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import helpers
+from oracle import spmm_oracle as so
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip(gpu):
+    gpu.lib()                                    # the HIP runtime the library itself uses
+    h = C.CDLL("libamdhip64.so.7")
+    for name in ("hipStreamCreate", "hipStreamDestroy", "hipStreamSynchronize", "hipStreamBeginCapture",
+                 "hipStreamEndCapture", "hipGraphInstantiate", "hipGraphLaunch", "hipGraphExecDestroy",
+                 "hipGraphDestroy"):
+        getattr(h, name).restype = C.c_int
+    return h
+
+
+def ok(rc):
+    assert rc == 0, f"HIP call failed with {rc}"
+
+
+def make_case(gpu, seed, N):
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=seed, n_long=6, zeros=7), seed=seed)
+    X = np.random.default_rng(seed).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    return g, X, op
+
+
+def test_two_streams_two_handles(gpu, hip):
+    s1, s2 = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(s1)))
+    ok(hip.hipStreamCreate(C.byref(s2)))
+    cases = [make_case(gpu, 31, 64), make_case(gpu, 32, 100)]
+    bufs = []
+    for (g, X, op), s in zip(cases, (s1, s2)):
+        dX, dY = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer(g.n_rows * X.shape[1] * 4)
+        dY.fill_u32(0x7FC00000)
+        bufs.append((dX, dY))
+    gpu._lib.check(gpu.lib().accel_stream_sync(None))
+    for _ in range(3):                                    # interleaved launches on both streams
+        for (g, X, op), (dX, dY), s in zip(cases, bufs, (s1, s2)):
+            op.run(dX, dY, X.shape[1], stream=s.value)
+    ok(hip.hipStreamSynchronize(s1))
+    ok(hip.hipStreamSynchronize(s2))
+    for (g, X, op), (dX, dY) in zip(cases, bufs):
+        Y = dY.to_numpy(np.float32, (g.n_rows, X.shape[1]))
+        assert so.check(Y, g.indptr, g.indices, g.values, X) <= so.TOL
+        dX.close(); dY.close(); op.close()
+    ok(hip.hipStreamDestroy(s1))
+    ok(hip.hipStreamDestroy(s2))
+
+
+def test_graph_capture_and_replay(gpu, hip):
+    g, X, op = make_case(gpu, 33, 64)
+    N = 64
+    dX, dY = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer(g.n_rows * N * 4)
+    op.run(dX, dY, N)                                     # eager warm-up: allocates the scratch for this N
+    op.synchronize()
+    eager = dY.to_numpy(np.float32, (g.n_rows, N))
+    s = C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(s)))
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamBeginCapture(s, 0))                   # hipStreamCaptureModeGlobal
+    op.run(dX, dY, N, stream=s.value)
+    ok(hip.hipStreamEndCapture(s, C.byref(graph)))
+    ok(hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0))
+    for rep in range(4):
+        dY.fill_u32(0x7FC00000)                           # eager work between replays
+        op.synchronize()
+        ok(hip.hipGraphLaunch(gexec, s))
+        ok(hip.hipStreamSynchronize(s))
+        Y = dY.to_numpy(np.float32, (g.n_rows, N))
+        assert np.array_equal(Y, eager), f"replay {rep} differs from the eager result"
+    ok(hip.hipGraphExecDestroy(gexec))
+    ok(hip.hipGraphDestroy(graph))
+    ok(hip.hipStreamDestroy(s))
+    dX.close(); dY.close(); op.close()
