@@ -190,6 +190,19 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall / a.steps * 1e3
 
+    # secondary figure: upstream's own protocol (spmm_base.h:44-60): 4 warm-up launches,
+    # then 4 launches each timed on the host clock around launch + synchronisation
+    for _ in range(4):
+        op.run(dX, dY, N)
+    op.synchronize()
+    ref_protocol = 0.0
+    for _ in range(4):
+        t1 = time.perf_counter()
+        op.run(dX, dY, N)
+        op.synchronize()
+        ref_protocol += time.perf_counter() - t1
+    ref_protocol_ms = ref_protocol / 4 * 1e3
+
     flops = 2.0 * g.nnz * N
     alg_bytes = g.nnz * 8 + g.n_cols * N * 4 + g.n_rows * N * 4
     main_avg_ms = float(np.mean(main_ms))
@@ -204,13 +217,15 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{a.workload}: {g.n_rows} rows, {g.nnz} non-zeros, N={N}",
                    "rows": g.n_rows, "nnz": g.nnz, "N": N, "blocks": int(info.n_blocks),
-                   "preprocess_ms": round(info.preprocess_ms, 2)},
+                   "preprocess_ms": round(info.preprocess_ms, 2),
+                   "reference_protocol_ms": round(ref_protocol_ms, 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": recorded_traffic(a.workload, N),
                      "kernel": "spmm_gather_kernel", "kernel_ms_avg": round(main_avg_ms, 5),
                      "kernel_ms_min": round(float(np.min(main_ms)), 5),
                      "all_kernels_ms_avg": round(float(np.mean(tot_ms)), 5),
+                     "all_kernels_ms_median": round(float(np.median(tot_ms)), 5),
                      "algorithmic_bytes": alg_bytes},
     }
 

@@ -506,6 +506,19 @@ int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream
     return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr);
 }
 
+int accel_run_epilogue(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias,
+                       int flags, void *stream)
+{
+    clear_error();
+    if (!h) { set_error("accel_run_epilogue: null handle"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_run_epilogue: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (N <= 0) { set_error("accel_run_epilogue: N must be positive, got %d", N); return ACCEL_ERR_ARG; }
+    if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("accel_run_epilogue: null dense operand"); return ACCEL_ERR_ARG; }
+    if (flags & ~ACCEL_EPILOGUE_RELU) { set_error("accel_run_epilogue: unknown flags %d", flags); return ACCEL_ERR_ARG; }
+    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, bias,
+                       (flags & ACCEL_EPILOGUE_RELU) ? 1 : 0);
+}
+
 int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup, int iters,
                float *ms_total, float *ms_main, void *stream)
 {

@@ -116,7 +116,8 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     const int4 *__restrict__ work, int n_units,
     const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
     const int32_t *__restrict__ perm, const float *__restrict__ X, float *__restrict__ Y,
-    float *__restrict__ partial, int N, int n_zero_rows, int n_entry_groups)
+    float *__restrict__ partial, int N, int n_zero_rows, int n_entry_groups,
+    const float *__restrict__ bias, int relu)
 {
     constexpr int G = 64 / L;        // lane groups per wavefront
     constexpr int CW = L * VEC;      // columns covered per pass
@@ -130,7 +131,9 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
             const int64_t r = i / N;
             const int64_t c = i - r * N;
             const int64_t out_row = perm ? perm[r] : r;
-            Y[out_row * N + c] = 0.0f;
+            float v = bias ? bias[c] : 0.0f;               // A X is 0 for this row
+            if (relu) v = fmaxf(v, 0.0f);
+            Y[out_row * N + c] = v;
         }
         return;
     }
@@ -264,8 +267,17 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
             if (live && k == 0) {
                 if (is_long)
                     store_vec<VEC>(partial + (int64_t)(deg - (kDegBound + 1)) * N + col, acc);
-                else
+                else {
+                    if (bias) {
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[v] += bias[col + v];
+                    }
+                    if (relu) {
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[v] = fmaxf(acc[v], 0.0f);
+                    }
                     store_out<VEC>(Y + out_row * N + col, acc);
+                }
             }
         }
     }
@@ -274,7 +286,8 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 // Adds the partial sums of each long row in slot order and writes the row.
 __global__ __launch_bounds__(kWgThreads) void long_row_reduce_kernel(
     const float *__restrict__ partial, const int32_t *__restrict__ long_slot,
-    const int32_t *__restrict__ perm, int64_t first_long_row, float *__restrict__ Y, int N)
+    const int32_t *__restrict__ perm, int64_t first_long_row, float *__restrict__ Y, int N,
+    const float *__restrict__ bias, int relu)
 {
     __shared__ float red[kWgThreads];
     const int64_t r = first_long_row + blockIdx.x;
@@ -296,6 +309,8 @@ __global__ __launch_bounds__(kWgThreads) void long_row_reduce_kernel(
         if (my_sg == 0 && c < N) {
             float t = acc;
             for (int q = 1; q < sg; q++) t += red[q * cw + c_in];
+            if (bias) t += bias[c];
+            if (relu) t = fmaxf(t, 0.0f);
             Y[out_row * N + c] = t;
         }
         __syncthreads();
@@ -318,13 +333,14 @@ __global__ __launch_bounds__(256) void copy_u32_kernel(uint32_t *__restrict__ ds
 template <int VEC>
 int launch_for_vec(int L, dim3 grid, hipStream_t s, const int4 *work, int n_units,
                    const int32_t *s_idx, const float *s_val, const int32_t *perm, const float *X,
-                   float *Y, float *partial, int N, int n_zero_rows, int n_entry_groups)
+                   float *Y, float *partial, int N, int n_zero_rows, int n_entry_groups,
+                   const float *bias, int relu)
 {
 #define ACCEL_LAUNCH(LL)                                                                      \
     case LL:                                                                                  \
         spmm_gather_kernel<LL, VEC><<<grid, dim3(kWgThreads), 0, s>>>(                        \
             work, n_units, s_idx, s_val, perm, X, Y, partial, N, n_zero_rows,                 \
-            n_entry_groups);                                                                  \
+            n_entry_groups, bias, relu);                                                                \
         break;
     switch (L) {
         ACCEL_LAUNCH(1)
@@ -364,7 +380,7 @@ int copy_u32(void *dst, const void *src, size_t n, hipStream_t s)
 }
 
 int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
-                hipEvent_t after_main)
+                hipEvent_t after_main, const float *bias, int relu)
 {
     if (h->rows == 0) return ACCEL_OK;
     // widest vector the row stride and the base pointers allow
@@ -403,19 +419,19 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         const int4 *wk = reinterpret_cast<const int4 *>(h->work);
         if (vec == 4)
             rc = launch_for_vec<4>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups);
+                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups, bias, relu);
         else if (vec == 2)
             rc = launch_for_vec<2>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups);
+                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups, bias, relu);
         else
             rc = launch_for_vec<1>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups);
+                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups, bias, relu);
         if (rc) return rc;
     }
     if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));
     if (h->n_long_rows > 0) {
         long_row_reduce_kernel<<<dim3((unsigned)h->n_long_rows), dim3(kWgThreads), 0, stream>>>(
-            h->partial, h->long_slot, h->perm, h->rows - h->n_long_rows, Y, N);
+            h->partial, h->long_slot, h->perm, h->rows - h->n_long_rows, Y, N, bias, relu);
     }
     ACCEL_HIP(hipGetLastError());
     return ACCEL_OK;

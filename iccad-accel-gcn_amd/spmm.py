@@ -111,6 +111,11 @@ class AccelSpMM:
         """One asynchronous launch; X, Y are device buffers."""
         check(lib().accel_run(self._h, ptr(X), ptr(Y), int(N), ptr(stream)))
 
+    def run_epilogue(self, X, Y, N: int, bias=None, relu=False, stream=None) -> None:
+        """Y = act(A X + bias) in one launch; bias is a device buffer of N floats or None."""
+        check(lib().accel_run_epilogue(self._h, ptr(X), ptr(Y), int(N), ptr(bias),
+                                       _lib.EPILOGUE_RELU if relu else 0, ptr(stream)))
+
     def synchronize(self, stream=None) -> None:
         check(lib().accel_stream_sync(ptr(stream)))
 

@@ -147,6 +147,15 @@ int accel_get_plan(const accel_handle *h, int32_t *out, int64_t cap_units, int64
  * hipStream_t, NULL = default stream); X and Y are device pointers. */
 int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream);
 
+/* run with the rest of a GCN layer fused into the store: Y = act(A X + bias).
+ * No counterpart upstream (its kernel stops at A X); this is the step a GCN layer
+ * applies right after the aggregation, done here while the row is in registers
+ * instead of as a second pass over Y.  bias: N floats on the device, or NULL.
+ * flags: 0 or ACCEL_EPILOGUE_RELU.  Rows of degree 0 receive act(bias). */
+#define ACCEL_EPILOGUE_RELU 1
+int accel_run_epilogue(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias,
+                       int flags, void *stream);
+
 /* Timing protocol of SPMM_BASE::timing_body (spmm_base.h:34-63) with HIP
  * events on `stream`: `warmup` untimed runs, then `iters` runs each bracketed
  * by events.  ms_total[i] covers everything accel_run launches; ms_main[i]

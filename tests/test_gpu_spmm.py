@@ -207,3 +207,84 @@ def test_medium_power_law_graph(gpu):
         R, S = c_oracle.spmm_csr_f64(g.indptr, g.indices, g.values, X)
         assert so.scaled_error(Y, R, S) <= TOL
     op.close()
+
+
+@pytest.mark.parametrize("N", [16, 64, 100, 3])
+def test_fused_bias_and_relu(gpu, mixed, N):
+    """Y = relu(A X + b) in the store; rows of degree 0 become relu(b)."""
+    g, op = mixed
+    rng = np.random.default_rng(N)
+    X = rng.uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    b = rng.uniform(-0.5, 0.5, N).astype(np.float32)
+    dX, db = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer.from_numpy(b)
+    dY = gpu.DeviceBuffer(g.n_rows * N * 4)
+    R, S = so.spmm_fp64(g.indptr, g.indices, g.values, X)
+    for bias, relu in ((db, True), (db, False), (None, True), (None, False)):
+        dY.fill_u32(0x7FC00000)
+        op.run_epilogue(dX, dY, N, bias=bias, relu=relu)
+        op.synchronize()
+        Y = dY.to_numpy(np.float32, (g.n_rows, N)).astype(np.float64)
+        ref = R + (b.astype(np.float64) if bias is not None else 0.0)
+        scale = S + (np.abs(b) if bias is not None else 0.0)
+        if relu:
+            ref = np.maximum(ref, 0.0)
+        assert np.isfinite(Y).all()
+        assert np.max(np.abs(Y - ref) / np.maximum(scale, np.finfo(np.float32).tiny)) <= TOL
+        if relu:
+            assert Y.min() >= 0.0
+    with pytest.raises(gpu.AccelError) as e:
+        gpu._lib.check(gpu.lib().accel_run_epilogue(op._h, gpu._lib.ptr(dX), gpu._lib.ptr(dY), N, None, 8, None))
+    assert e.value.status == gpu._lib.ERR_ARG
+    for buf in (dX, db, dY):
+        buf.close()
+
+
+def test_operands_beyond_4_gib(gpu):
+    """X and Y larger than 4 GiB: row offsets need 64-bit arithmetic.  The
+    matrix references rows of X at both ends of a 5.1 GB buffer and writes rows
+    of Y at both ends of a 4.4 GB buffer; only the touched rows travel to the host."""
+    import ctypes as C
+    N, n_cols, n_rows = 256, 5_000_000, 4_300_000
+    rng = np.random.default_rng(0)
+    cols = np.unique(np.concatenate([[0, 1, n_cols - 1, n_cols - 2, 4_194_304, 4_194_303],
+                                     rng.integers(0, n_cols, 500)])).astype(np.int32)
+    live_rows = np.unique(np.concatenate([[0, 7, n_rows - 1, n_rows - 2, 4_194_304, 4_194_305],
+                                          rng.integers(0, n_rows, 60)]))
+    deg = np.zeros(n_rows, dtype=np.int64)
+    deg[live_rows] = rng.integers(1, 40, live_rows.size)
+    deg[live_rows[3]] = 450                                   # one long row as well
+    indptr = np.zeros(n_rows + 1, dtype=np.int64)
+    np.cumsum(deg, out=indptr[1:])
+    nnz = int(indptr[-1])
+    idx = np.concatenate([np.sort(rng.choice(cols, d, replace=False)) for d in deg[live_rows]]).astype(np.int32)
+    val = rng.uniform(-1, 1, nnz).astype(np.float32)
+    Xrows = rng.uniform(-1, 1, (cols.size, N)).astype(np.float32)
+
+    lib = gpu.lib()
+    dX = gpu.DeviceBuffer(n_cols * N * 4)
+    dY = gpu.DeviceBuffer(n_rows * N * 4)
+    dX.fill_u32(0)
+    dY.fill_u32(0x7FC00000)
+    for c, row in zip(cols, Xrows):                            # only the referenced rows of X are non-zero
+        gpu._lib.check(lib.accel_memcpy_h2d(C.c_void_p(dX.address + int(c) * N * 4), C.c_void_p(row.ctypes.data), N * 4))
+    op = gpu.AccelSpMM(indptr.astype(np.int32), idx, val, n_cols).preprocess()
+    op.run(dX, dY, N)
+    op.synchronize()
+
+    def y_row(r):
+        out = np.empty(N, dtype=np.float32)
+        gpu._lib.check(lib.accel_memcpy_d2h(C.c_void_p(out.ctypes.data), C.c_void_p(dY.address + int(r) * N * 4), N * 4))
+        return out
+
+    pos = {int(c): i for i, c in enumerate(cols)}
+    for r in live_rows:
+        a, b = indptr[r], indptr[r + 1]
+        xs = Xrows[[pos[int(c)] for c in idx[a:b]]].astype(np.float64)
+        ref = (val[a:b].astype(np.float64)[:, None] * xs).sum(0)
+        scale = (np.abs(val[a:b]).astype(np.float64)[:, None] * np.abs(xs)).sum(0)
+        assert np.max(np.abs(y_row(r) - ref) / np.maximum(scale, 1e-30)) <= TOL, r
+    live = set(live_rows.tolist())
+    for r in (1, 2, 4_194_303, 4_194_306, n_rows - 3, n_rows // 2):     # zero-degree rows at both ends
+        if r not in live:
+            assert np.array_equal(y_row(r), np.zeros(N, np.float32)), r
+    op.close(); dX.close(); dY.close()
