@@ -15,7 +15,10 @@ constexpr int kDegBound = ACCEL_DEG_BOUND;            // non-zeros per block4 en
 constexpr int kSlices = ACCEL_SLICES_PER_BLOCK;       // slices per entry (metadata ABI)
 constexpr int kSliceNz = kDegBound / kSlices;         // 32
 constexpr int kXcds = 8;                              // accelerator dies, each with its own L2
-constexpr int kWavesPerGroup = 4;                     // wavefronts (work units) per workgroup
+#ifndef ACCEL_WAVES_PER_GROUP
+#define ACCEL_WAVES_PER_GROUP 4
+#endif
+constexpr int kWavesPerGroup = ACCEL_WAVES_PER_GROUP; // wavefronts (work units) per workgroup
 
 // Column group of a non-zero: which die's L2 should hold that row of X.  Eight
 // consecutive columns share a group so that neighbouring short rows of X (one

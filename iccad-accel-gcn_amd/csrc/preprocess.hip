@@ -831,6 +831,10 @@ int preprocess_device(accel_handle *h)
     ACCEL_HIP(hipStreamSynchronize(s));
     h->block4 = b4;
     h->n_blocks = nb;
+    if (nb + (int64_t)kXcds * (n_long + kWavesPerGroup) > (int64_t)INT_MAX) {
+        set_error("the launch plan would exceed 2^31 work units (%lld block4 entries)", (long long)nb);
+        return ACCEL_ERR_ARG;
+    }
 
     // ---- work list ------------------------------------------------------------
     if ((rc = build_work_list(h, gcount.as<int>(), sip.as<int32_t>(), first_long, s))) return rc;

@@ -32,7 +32,11 @@ namespace {
 
 constexpr int kWaves = kWavesPerGroup;    // wavefronts (= work units) per workgroup
 constexpr int kWgThreads = 64 * kWaves;
-constexpr int kZeroFloats = 16384;        // floats zero-filled per extra workgroup
+constexpr int kZeroFloats = 8192;         // floats zero-filled per extra workgroup
+
+// zero-degree rows handled by one zero-fill workgroup (N is a multiple of VEC, so
+// a workgroup's share is a whole number of vectors)
+__host__ __device__ inline int zero_rows_per_group(int N) { return N >= kZeroFloats ? 1 : kZeroFloats / N; }
 
 // build-time tuning knobs (defaults are the measured best)
 #ifndef ACCEL_UNROLL
@@ -116,31 +120,36 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     const int4 *__restrict__ work, int n_units,
     const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
     const int32_t *__restrict__ perm, const float *__restrict__ X, float *__restrict__ Y,
-    float *__restrict__ partial, int N, int n_zero_rows, int n_entry_groups,
+    float *__restrict__ partial, int N, int n_zero_rows, int n_zero_groups,
     const float *__restrict__ bias, int relu)
 {
     constexpr int G = 64 / L;        // lane groups per wavefront
     constexpr int CW = L * VEC;      // columns covered per pass
     __shared__ int2 stage[kWaves][kDegBound];
 
-    if ((int)blockIdx.x >= n_entry_groups) {
-        // zero-degree rows: they are the first n_zero_rows rows of the sorted order
-        const int64_t first = (int64_t)(blockIdx.x - n_entry_groups) * kZeroFloats;
-        const int64_t total = (int64_t)n_zero_rows * N;
-        for (int64_t i = first + threadIdx.x; i < first + kZeroFloats && i < total; i += kWgThreads) {
-            const int64_t r = i / N;
-            const int64_t c = i - r * N;
-            const int64_t out_row = perm ? perm[r] : r;
-            float v = bias ? bias[c] : 0.0f;               // A X is 0 for this row
-            if (relu) v = fmaxf(v, 0.0f);
-            Y[out_row * N + c] = v;
+    if ((int)blockIdx.x < n_zero_groups) {
+        // zero-degree rows: they are the first n_zero_rows rows of the sorted order.
+        // These workgroups come first in the grid so that they do not form a tail.
+        const int rows_here = zero_rows_per_group(N);
+        const int r0 = (int)blockIdx.x * rows_here;
+        const int n = min(rows_here, n_zero_rows - r0) * N;        // floats of this workgroup
+        float fill[VEC];
+        for (int i = (int)threadIdx.x * VEC; i < n; i += kWgThreads * VEC) {
+            const int r = i / N, c = i - r * N;
+            const int64_t out_row = perm ? perm[r0 + r] : r0 + r;
+#pragma unroll
+            for (int v = 0; v < VEC; v++) {
+                float t = bias ? bias[c + v] : 0.0f;                // A X is 0 for this row
+                fill[v] = relu ? fmaxf(t, 0.0f) : t;
+            }
+            store_out<VEC>(Y + out_row * N + c, fill);
         }
         return;
     }
 
     const int lane = threadIdx.x & 63;
     const int wv = uniform(threadIdx.x >> 6);
-    const int e = (int)blockIdx.x * kWaves + wv;
+    const int e = ((int)blockIdx.x - n_zero_groups) * kWaves + wv;
     if (e >= n_units) return;
 
     const int4 b = work[e];
@@ -333,14 +342,14 @@ __global__ __launch_bounds__(256) void copy_u32_kernel(uint32_t *__restrict__ ds
 template <int VEC>
 int launch_for_vec(int L, dim3 grid, hipStream_t s, const int4 *work, int n_units,
                    const int32_t *s_idx, const float *s_val, const int32_t *perm, const float *X,
-                   float *Y, float *partial, int N, int n_zero_rows, int n_entry_groups,
+                   float *Y, float *partial, int N, int n_zero_rows, int n_zero_groups,
                    const float *bias, int relu)
 {
 #define ACCEL_LAUNCH(LL)                                                                      \
     case LL:                                                                                  \
         spmm_gather_kernel<LL, VEC><<<grid, dim3(kWgThreads), 0, s>>>(                        \
             work, n_units, s_idx, s_val, perm, X, Y, partial, N, n_zero_rows,                 \
-            n_entry_groups, bias, relu);                                                                \
+            n_zero_groups, bias, relu);                                                                  \
         break;
     switch (L) {
         ACCEL_LAUNCH(1)
@@ -407,7 +416,11 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         }
     }
     const int64_t entry_groups = h->n_units / kWaves;
-    const int64_t zero_groups = (h->n_zero_rows * (int64_t)N + kZeroFloats - 1) / kZeroFloats;
+    // zero-fill workgroups come first; their count is rounded up to a multiple of the
+    // die count so that entry group i still lands on die i % 8 (surplus ones exit at once)
+    const int zr = zero_rows_per_group(N);
+    int64_t zero_groups = (h->n_zero_rows + zr - 1) / zr;
+    zero_groups = (zero_groups + kXcds - 1) / kXcds * kXcds;
     const int64_t groups = entry_groups + zero_groups;
     if (groups > 0x7fffffffLL) {
         set_error("launch of %lld workgroups exceeds the grid limit", (long long)groups);
@@ -419,13 +432,13 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         const int4 *wk = reinterpret_cast<const int4 *>(h->work);
         if (vec == 4)
             rc = launch_for_vec<4>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups, bias, relu);
+                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)zero_groups, bias, relu);
         else if (vec == 2)
             rc = launch_for_vec<2>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups, bias, relu);
+                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)zero_groups, bias, relu);
         else
             rc = launch_for_vec<1>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)entry_groups, bias, relu);
+                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)zero_groups, bias, relu);
         if (rc) return rc;
     }
     if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));

@@ -288,3 +288,27 @@ def test_operands_beyond_4_gib(gpu):
         if r not in live:
             assert np.array_equal(y_row(r), np.zeros(N, np.float32)), r
     op.close(); dX.close(); dY.close()
+
+
+def test_random_shapes(gpu):
+    """Sixty seeded random matrices: random row counts, degree mixes (empty rows,
+    every slice-table regime, rows of several thousand non-zeros) and column
+    counts 1..320, rectangular as well as square."""
+    rng = np.random.default_rng(2024)
+    pool = np.array([0, 0, 1, 1, 2, 3, 7, 12, 31, 32, 33, 64, 65, 96, 97, 128, 129, 191, 192, 200, 383, 384,
+                     385, 500, 768, 769, 1153, 3000])
+    for case in range(60):
+        n_rows = int(rng.integers(1, 260))
+        deg = rng.choice(pool, size=n_rows, p=None)
+        if case % 3 == 0:
+            deg = np.minimum(deg, 40)                         # short rows only
+        n_cols = int(max(deg.max() + 1, rng.integers(1, 5000)))
+        N = int(rng.integers(1, 321))
+        g = gpu.synthetic.random_csr(n_rows, n_cols, deg, seed=case)
+        X = rng.uniform(-1, 1, (n_cols, N)).astype(np.float32)
+        op = gpu.AccelSpMM(g.indptr, g.indices, g.values, n_cols).preprocess()
+        Y = op.matmul(X)
+        assert np.isfinite(Y).all(), (case, n_rows, N)
+        err = so.check(Y, g.indptr, g.indices, g.values, X)
+        assert err <= TOL, (case, n_rows, n_cols, N, err)
+        op.close()
