@@ -311,8 +311,17 @@ __global__ __launch_bounds__(kWgThreads) void long_row_reduce_kernel(
     for (int c0 = 0; c0 < N; c0 += cw) {
         const int c = c0 + c_in;
         float acc = 0.0f;
-        if (c < N)
-            for (int sgm = my_sg; sgm < nseg; sgm += sg) acc += src[(int64_t)sgm * N + c];
+        if (c < N) {
+            int sgm = my_sg;
+            for (; sgm + 7 * sg < nseg; sgm += 8 * sg) {       // eight loads in flight, added in order
+                float t[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) t[u] = src[(int64_t)(sgm + u * sg) * N + c];
+#pragma unroll
+                for (int u = 0; u < 8; u++) acc += t[u];
+            }
+            for (; sgm < nseg; sgm += sg) acc += src[(int64_t)sgm * N + c];
+        }
         red[threadIdx.x] = acc;
         __syncthreads();
         if (my_sg == 0 && c < N) {
