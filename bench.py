@@ -231,10 +231,13 @@ def main():
 
     if a.compare_rocsparse:
         rs, Yr = rocsparse_baseline(pkg, op, g, dX, N)
+        # our side measured the same way: two events around each run, nothing in between
+        ours, _ = op.time(dX, dY, N, warmup=3, iters=10, split=False)
+        ours_ms = float(np.median(ours))
         Ymine = dY.to_numpy(np.float32, (g.n_rows, N))
         best = min((v["ms"] for v in rs.values() if "ms" in v), default=None)
-        result["rocsparse"] = {"algorithms": rs, "best_ms": best,
-                               "speedup_vs_best": round(best / float(np.mean(tot_ms)), 3) if best else None,
+        result["rocsparse"] = {"algorithms": rs, "best_ms": best, "ours_ms": round(ours_ms, 5),
+                               "speedup_vs_best": round(best / ours_ms, 3) if best else None,
                                "max_abs_diff_vs_last_alg": float(np.max(np.abs(Ymine - Yr))) if Yr.size else 0.0}
     if not a.no_cpu:
         base, n_rows, Yc = cpu_baseline(g, X, N)

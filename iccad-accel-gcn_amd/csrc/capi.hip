@@ -345,6 +345,18 @@ int accel_destroy(accel_handle *h)
     return ACCEL_OK;
 }
 
+int accel_set_plan_unit(accel_handle *h, int unit_nz)
+{
+    clear_error();
+    if (!h) { set_error("accel_set_plan_unit: null handle"); return ACCEL_ERR_ARG; }
+    if (unit_nz != 0 && (unit_nz < 16 || unit_nz > kDegBound)) {
+        set_error("accel_set_plan_unit: unit must be 0 (automatic) or 16..384, got %d", unit_nz);
+        return ACCEL_ERR_ARG;
+    }
+    h->plan_unit_option = unit_nz;
+    return ACCEL_OK;
+}
+
 int accel_preprocess(accel_handle *h)
 {
     clear_error();
@@ -365,6 +377,10 @@ int accel_get_info(const accel_handle *h, accel_info *out)
     out->n_long_rows = h->n_long_rows; out->n_zero_rows = h->n_zero_rows;
     out->max_degree = h->max_degree; out->already_sorted = h->identity_perm ? 1 : 0;
     out->preprocess_ms = h->preprocess_ms;
+    out->n_plan_units = h->n_units;
+    out->n_split_rows = h->n_split_rows;
+    out->plan_unit_nz = h->plan_unit;
+    out->reserved = 0;
     return ACCEL_OK;
 }
 

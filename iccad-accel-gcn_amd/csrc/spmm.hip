@@ -451,9 +451,9 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         if (rc) return rc;
     }
     if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));
-    if (h->n_long_rows > 0) {
-        long_row_reduce_kernel<<<dim3((unsigned)h->n_long_rows), dim3(kWgThreads), 0, stream>>>(
-            h->partial, h->long_slot, h->perm, h->rows - h->n_long_rows, Y, N, bias, relu);
+    if (h->n_split_rows > 0) {
+        long_row_reduce_kernel<<<dim3((unsigned)h->n_split_rows), dim3(kWgThreads), 0, stream>>>(
+            h->partial, h->long_slot, h->perm, h->rows - h->n_split_rows, Y, N, bias, relu);
     }
     ACCEL_HIP(hipGetLastError());
     return ACCEL_OK;

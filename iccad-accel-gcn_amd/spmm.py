@@ -59,7 +59,11 @@ class AccelSpMM:
         self._info = None
 
     # -- preprocess ---------------------------------------------------------
-    def preprocess(self) -> "AccelSpMM":
+    def preprocess(self, plan_unit: int | None = None) -> "AccelSpMM":
+        """Degree sort, block4 metadata and launch plan on the GPU.  ``plan_unit``
+        (16..384) overrides the automatic choice of non-zeros per wavefront."""
+        if plan_unit is not None:
+            check(lib().accel_set_plan_unit(self._h, int(plan_unit)))
         check(lib().accel_preprocess(self._h))
         info = Info()
         check(lib().accel_get_info(self._h, C.byref(info)))
@@ -135,12 +139,15 @@ class AccelSpMM:
             dX.close()
             dY.close()
 
-    def time(self, X, Y, N: int, warmup: int = 4, iters: int = 20, stream=None):
-        """HIP-event timings in ms: (total per run, gather kernel only)."""
+    def time(self, X, Y, N: int, warmup: int = 4, iters: int = 20, stream=None, split: bool = True):
+        """HIP-event timings in ms: (total per run, gather kernel only).  With
+        ``split=False`` no event is recorded between the two kernels of a run (the
+        second array is then all zeros); use that for launches of a few microseconds,
+        where the extra event is a visible part of the total."""
         tot = np.zeros(iters, dtype=np.float32)
         main = np.zeros(iters, dtype=np.float32)
         check(lib().accel_time(self._h, ptr(X), ptr(Y), int(N), warmup, iters,
-                               ptr(tot, C.c_float), ptr(main, C.c_float), ptr(stream)))
+                               ptr(tot, C.c_float), ptr(main, C.c_float) if split else None, ptr(stream)))
         return tot, main
 
     def close(self) -> None:

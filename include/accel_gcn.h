@@ -106,6 +106,14 @@ int accel_create(const int32_t *indptr, const int32_t *idx, const float *val, in
  * sorted), gathers the permuted CSR, and builds the block4 metadata. */
 int accel_preprocess(accel_handle *h);
 
+/* Granularity of the launch plan (no counterpart upstream, whose unit is always one
+ * block4 entry): the most non-zeros one wavefront takes, 16..384, or 0 to let the
+ * library choose from the size of the matrix (the default).  Rows with more
+ * non-zeros are cut into pieces added up through partial sums; block4 entries
+ * of shorter rows are cut into units of whole rows.  The block4 metadata itself
+ * never changes.  Call before accel_preprocess. */
+int accel_set_plan_unit(accel_handle *h, int unit_nz);
+
 /* Check externally produced metadata (a .block4 file) against what
  * accel_preprocess built for this CSR; ACCEL_ERR_META if any int differs. */
 int accel_check_block4(accel_handle *h, const int32_t *block4_host, int64_t n_blocks);
@@ -119,6 +127,10 @@ typedef struct accel_info {
     int32_t max_degree;
     int32_t already_sorted; /* 1: input rows were already in ascending degree order */
     double preprocess_ms;   /* wall time of the last accel_preprocess */
+    int64_t n_plan_units;   /* wavefronts of one launch (launch plan, incl. padding) */
+    int64_t n_split_rows;   /* rows cut into pieces that go through partial sums */
+    int32_t plan_unit_nz;   /* most non-zeros one wavefront takes (<= 384) */
+    int32_t reserved;
 } accel_info;
 int accel_get_info(const accel_handle *h, accel_info *out);
 

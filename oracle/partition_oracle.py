@@ -213,13 +213,14 @@ def column_group(col):
     return (np.asarray(col) >> 3) & (N_COLUMN_GROUPS - 1)
 
 
-def group_long_rows(indptr, indices, values):
-    """Stable partition of the non-zeros of every row with degree > 384 by
+def group_long_rows(indptr, indices, values, threshold=DEG_BOUND):
+    """Stable partition of the non-zeros of every row with degree > threshold
+    (the launch plan's unit size, 384 unless the plan uses smaller units) by
     column_group(); all other rows are left as they are."""
     indptr = np.asarray(indptr, dtype=np.int64)
     indices = np.array(indices, copy=True)
     values = None if values is None else np.array(values, copy=True)
-    for r in np.flatnonzero(np.diff(indptr) > DEG_BOUND):
+    for r in np.flatnonzero(np.diff(indptr) > threshold):
         a, b = indptr[r], indptr[r + 1]
         order = np.argsort(column_group(indices[a:b]), kind="stable")
         indices[a:b] = indices[a:b][order]

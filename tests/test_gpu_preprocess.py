@@ -46,9 +46,12 @@ def test_stage_on_gpu_writes_golden_file(gpu, tmp_path):
         assert (tmp_path / "meta" / f"{name}.block4").read_bytes() == block4_codec.load(name).tobytes()
 
 
-def check_preprocess(gpu, g):
-    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
-    perm, sip, six, sval, b4 = helpers.expected_preprocess(g.indptr, g.indices, g.values)
+def check_preprocess(gpu, g, plan_unit=None):
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_unit)
+    if plan_unit is not None:
+        assert op.info.plan_unit_nz == plan_unit
+    perm, sip, six, sval, b4 = helpers.expected_preprocess(g.indptr, g.indices, g.values,
+                                                           op.info.plan_unit_nz)
     assert np.array_equal(op.perm(), perm)
     ip, ix, v = op.sorted_csr()
     assert np.array_equal(ip, sip) and np.array_equal(ix, six) and np.array_equal(v, sval)
@@ -60,6 +63,7 @@ def check_preprocess(gpu, g):
     assert info.n_zero_rows == int((d == 0).sum()) and info.n_long_rows == int((d > 384).sum())
     assert info.n_long_blocks == int(np.sum(-(-d[d > 384] // 384)))
     assert info.max_degree == int(d.max(initial=0))
+    assert info.n_split_rows == int((d > info.plan_unit_nz).sum())
     op.check_block4(b4)
     return op
 
@@ -96,7 +100,7 @@ def test_already_sorted_input(gpu, n_long):
     assert np.array_equal(op.perm(), np.arange(g0.n_rows))
     assert np.array_equal(op.block4(), po.partition_closed_form(sip))
     ip, ix, v = op.sorted_csr()
-    gix, gval = po.group_long_rows(sip, six, sval)
+    gix, gval = po.group_long_rows(sip, six, sval, op.info.plan_unit_nz)
     assert np.array_equal(ip, sip) and np.array_equal(ix, gix) and np.array_equal(v, gval)
     op.close()
 
@@ -173,24 +177,36 @@ def test_call_order_and_arguments(gpu):
 
 
 def check_plan(op, n_cols):
-    """The launch plan covers every non-zero exactly once, keeps block4 entries of
-    short rows verbatim, and queues each piece of a long row on the die that owns
-    its column group."""
+    """The launch plan covers every non-zero exactly once; units of whole rows stay
+    inside one block4 entry and hold at most plan_unit non-zeros (or one row); pieces of
+    split rows hold at most plan_unit non-zeros of one column group and are queued on the
+    die that owns that group."""
+    unit = op.info.plan_unit_nz
     plan = op.plan().astype(np.int64)
     b4 = op.block4().astype(np.int64)
     sip, six, _ = op.sorted_csr()
-    assert plan.shape[0] % 32 == 0                       # 8 queues x 4 wavefronts
+    deg = np.diff(sip)
+    assert plan.shape[0] % 32 == 0 and plan.shape[0] == op.info.n_plan_units      # 8 queues x 4 wavefronts
     live = plan[plan[:, 3] != 0]
     short = live[live[:, 0] <= 384]
     long_ = live[live[:, 0] > 384]
-    b4_short = b4[b4[:, 0] <= 384]
-    assert sorted(map(tuple, short)) == sorted(map(tuple, b4_short))
     covered = np.zeros(six.size, dtype=np.int32)
     for x, y, z, w in long_:
         covered[z:z + w] += 1
-        assert 0 < w <= 384 and sip[y] <= z and z + w <= sip[y + 1]
+        assert 0 < w <= unit and sip[y] <= z and z + w <= sip[y + 1] and deg[y] > unit
+    entry_of_row = {}
+    for d, r, loc, info in b4[b4[:, 0] <= 384]:
+        for q in range(info & 0xFFFF):
+            entry_of_row[r + q] = (d, r, loc, info >> 16)
     for d, r, loc, info in short:
-        covered[loc:loc + d * (info & 0xFFFF)] += 1
+        n = info & 0xFFFF
+        covered[loc:loc + d * n] += 1
+        assert d <= unit and (n * d <= unit or n == 1)
+        ed, er, eloc, ew = entry_of_row[r]                       # same block4 entry, same fields
+        assert ed == d and loc == sip[r] and (info >> 16) == ew
+        assert entry_of_row[r + n - 1][1] == er
+    if unit == 384:
+        assert sorted(map(tuple, short)) == sorted(map(tuple, b4[b4[:, 0] <= 384]))   # entries verbatim
     assert np.all(covered == 1)
     # queue of unit e is (e // 4) % 8
     queue = (np.arange(plan.shape[0]) // 4) % 8
@@ -202,10 +218,9 @@ def check_plan(op, n_cols):
     assert sorted(slots.tolist()) == list(range(len(long_)))
     order = np.argsort(slots)
     assert np.all(np.diff(long_[order, 1]) >= 0)
-    # queues are balanced to within one workgroup
     per_queue = [int((plan[queue == q][:, 3] != 0).sum()) for q in range(8)]
     if len(long_) == 0:
-        assert max(per_queue) - min(per_queue) <= 1
+        assert max(per_queue) - min(per_queue) <= 1               # queues are level
 
 
 @pytest.mark.parametrize("seed,n_long", [(0, 0), (1, 3), (2, 9)])
@@ -221,3 +236,22 @@ def test_launch_plan_hub_graph(gpu):
     op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
     check_plan(op, g.n_cols)
     op.close()
+
+
+@pytest.mark.parametrize("unit", [16, 50, 96, 200, 384])
+def test_plan_unit_sizes(gpu, unit):
+    """Smaller units change the plan and which rows are stored grouped, never the
+    block4 metadata or the product."""
+    from oracle import spmm_oracle as so
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=6, n_long=5), seed=6)
+    op = check_preprocess(gpu, g, plan_unit=unit)
+    check_plan(op, g.n_cols)
+    for N in (64, 10):
+        X = np.random.default_rng(unit + N).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+        Y = op.matmul(X)
+        assert np.isfinite(Y).all()
+        assert so.check(Y, g.indptr, g.indices, g.values, X) <= so.TOL
+    op.close()
+    with pytest.raises(gpu.AccelError) as e:
+        gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_unit=1000)
+    assert e.value.status == gpu._lib.ERR_ARG
