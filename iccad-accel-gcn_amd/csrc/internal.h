@@ -81,6 +81,7 @@ struct accel_handle {
     int plan_unit_option = 0;         // 0: choose from the size of the matrix
     int plan_unit = ACCEL_DEG_BOUND;
     int64_t n_split_rows = 0;         // rows with more than plan_unit non-zeros
+    int64_t n_big_rows = 0;           // of those, rows with more than 32 * plan_unit
     int64_t n_blocks = 0, n_long_blocks = 0, n_long_rows = 0, n_zero_rows = 0;
     int32_t max_degree = 0;
     double preprocess_ms = 0.0;

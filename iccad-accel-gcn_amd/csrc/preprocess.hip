@@ -152,6 +152,7 @@ struct Stats {
     int n_long_rows;
     int n_long_blocks;
     int n_split_rows;   // rows with more non-zeros than the plan's unit size
+    int n_big_rows;     // rows with more than 32 units' worth of non-zeros
 };
 
 __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restrict__ indptr,
@@ -160,8 +161,8 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
                                                           Stats *__restrict__ st, int split_deg)
 {
     // grid-stride over rows; one set of atomics per workgroup
-    __shared__ int part[kThreads / 64][7];
-    int bad = 0, unsorted = 0, dmax = 0, zero = 0, lrow = 0, lblk = 0, srow = 0;
+    __shared__ int part[kThreads / 64][8];
+    int bad = 0, unsorted = 0, dmax = 0, zero = 0, lrow = 0, lblk = 0, srow = 0, brow = 0;
     for (int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x; r < rows;
          r += (int64_t)gridDim.x * kThreads) {
         const int a = indptr[r], b = indptr[r + 1];
@@ -177,6 +178,7 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
         zero += d == 0;
         if (d > kDegBound) { lrow++; lblk += (d + kDegBound - 1) / kDegBound; }
         srow += d > split_deg;
+        brow += d > 32 * split_deg;
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -187,17 +189,18 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
         lrow += __shfl_xor(lrow, off);
         lblk += __shfl_xor(lblk, off);
         srow += __shfl_xor(srow, off);
+        brow += __shfl_xor(brow, off);
     }
     const int w = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) {
         part[w][0] = bad; part[w][1] = unsorted; part[w][2] = dmax;
-        part[w][3] = zero; part[w][4] = lrow; part[w][5] = lblk; part[w][6] = srow;
+        part[w][3] = zero; part[w][4] = lrow; part[w][5] = lblk; part[w][6] = srow; part[w][7] = brow;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int q = 1; q < kThreads / 64; q++) {
             bad |= part[q][0]; unsorted |= part[q][1]; dmax = max(dmax, part[q][2]);
-            zero += part[q][3]; lrow += part[q][4]; lblk += part[q][5]; srow += part[q][6];
+            zero += part[q][3]; lrow += part[q][4]; lblk += part[q][5]; srow += part[q][6]; brow += part[q][7];
         }
         if (bad) atomicOr(&st->bad_indptr, 1);
         if (unsorted) atomicOr(&st->unsorted, 1);
@@ -206,6 +209,7 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
         if (lrow) atomicAdd(&st->n_long_rows, lrow);
         if (lblk) atomicAdd(&st->n_long_blocks, lblk);
         if (srow) atomicAdd(&st->n_split_rows, srow);
+        if (brow) atomicAdd(&st->n_big_rows, brow);
     }
 }
 
@@ -780,7 +784,7 @@ int preprocess_device(accel_handle *h)
     h->n_blocks = h->n_long_blocks = h->n_long_rows = h->n_zero_rows = 0;
     h->max_degree = 0;
     h->n_units = h->n_long_units = 0;
-    h->n_split_rows = 0;
+    h->n_split_rows = h->n_big_rows = 0;
     h->plan_unit = h->plan_unit_option > 0 ? h->plan_unit_option : choose_plan_unit(rows, nnz);
     if (rows == 0) {
         h->identity_perm = true;
@@ -816,6 +820,7 @@ int preprocess_device(accel_handle *h)
     h->n_long_rows = hs.n_long_rows;
     h->n_long_blocks = hs.n_long_blocks;
     h->n_split_rows = hs.n_split_rows;
+    h->n_big_rows = hs.n_big_rows;
     h->identity_perm = !hs.unsorted;
 
     // ---- degree sort ------------------------------------------------------

@@ -33,6 +33,7 @@ namespace {
 constexpr int kWaves = kWavesPerGroup;    // wavefronts (= work units) per workgroup
 constexpr int kWgThreads = 64 * kWaves;
 constexpr int kZeroFloats = 8192;         // floats zero-filled per extra workgroup
+constexpr int kReduceThreads = 256;       // workgroup of the partial-sum reduction
 
 // zero-degree rows handled by one zero-fill workgroup (N is a multiple of VEC, so
 // a workgroup's share is a whole number of vectors)
@@ -292,44 +293,51 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     }
 }
 
-// Adds the partial sums of each long row in slot order and writes the row.
-__global__ __launch_bounds__(kWgThreads) void long_row_reduce_kernel(
+// Adds the partial sums of each split row in slot order and writes the row.
+// RPW rows share a 256-thread workgroup (256 / RPW threads each): rows with few
+// slots and few columns do not need a whole workgroup.
+template <int RPW>
+__global__ __launch_bounds__(kReduceThreads) void long_row_reduce_kernel(
     const float *__restrict__ partial, const int32_t *__restrict__ long_slot,
-    const int32_t *__restrict__ perm, int64_t first_long_row, float *__restrict__ Y, int N,
-    const float *__restrict__ bias, int relu)
+    const int32_t *__restrict__ perm, int64_t first_split_row, int lr_begin, int lr_end,
+    float *__restrict__ Y, int N, const float *__restrict__ bias, int relu)
 {
-    __shared__ float red[kWgThreads];
-    const int64_t r = first_long_row + blockIdx.x;
-    const int first = long_slot[blockIdx.x];
-    const int nseg = long_slot[blockIdx.x + 1] - first;
+    constexpr int T = kReduceThreads / RPW;        // threads per row
+    __shared__ float red[kReduceThreads];
+    const int sub_row = threadIdx.x / T, t = threadIdx.x % T;
+    const int lr = lr_begin + (int)blockIdx.x * RPW + sub_row;
+    const bool row_ok = lr < lr_end;
+    const int first = row_ok ? long_slot[lr] : 0;
+    const int nseg = row_ok ? long_slot[lr + 1] - first : 0;
     const float *src = partial + (int64_t)first * N;
-    const int64_t out_row = perm ? perm[r] : r;
-    int cw = 1;                                   // columns per pass: power of two <= 256
-    while (cw < N && cw < kWgThreads) cw <<= 1;
-    const int sg = kWgThreads / cw;               // slot groups
-    const int c_in = threadIdx.x % cw, my_sg = threadIdx.x / cw;
+    const int64_t r = first_split_row + lr;
+    const int64_t out_row = row_ok ? (perm ? perm[r] : r) : 0;
+    int cw = 1;                                    // columns per pass: power of two <= T
+    while (cw < N && cw < T) cw <<= 1;
+    const int sg = T / cw;                         // slot groups
+    const int c_in = t % cw, my_sg = t / cw;
     for (int c0 = 0; c0 < N; c0 += cw) {
         const int c = c0 + c_in;
         float acc = 0.0f;
         if (c < N) {
             int sgm = my_sg;
             for (; sgm + 7 * sg < nseg; sgm += 8 * sg) {       // eight loads in flight, added in order
-                float t[8];
+                float v[8];
 #pragma unroll
-                for (int u = 0; u < 8; u++) t[u] = src[(int64_t)(sgm + u * sg) * N + c];
+                for (int u = 0; u < 8; u++) v[u] = src[(int64_t)(sgm + u * sg) * N + c];
 #pragma unroll
-                for (int u = 0; u < 8; u++) acc += t[u];
+                for (int u = 0; u < 8; u++) acc += v[u];
             }
             for (; sgm < nseg; sgm += sg) acc += src[(int64_t)sgm * N + c];
         }
         red[threadIdx.x] = acc;
         __syncthreads();
-        if (my_sg == 0 && c < N) {
-            float t = acc;
-            for (int q = 1; q < sg; q++) t += red[q * cw + c_in];
-            if (bias) t += bias[c];
-            if (relu) t = fmaxf(t, 0.0f);
-            Y[out_row * N + c] = t;
+        if (row_ok && my_sg == 0 && c < N) {
+            float sum = acc;
+            for (int q = 1; q < sg; q++) sum += red[sub_row * T + q * cw + c_in];
+            if (bias) sum += bias[c];
+            if (relu) sum = fmaxf(sum, 0.0f);
+            Y[out_row * N + c] = sum;
         }
         __syncthreads();
     }
@@ -452,8 +460,24 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     }
     if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));
     if (h->n_split_rows > 0) {
-        long_row_reduce_kernel<<<dim3((unsigned)h->n_split_rows), dim3(kWgThreads), 0, stream>>>(
-            h->partial, h->long_slot, h->perm, h->rows - h->n_split_rows, Y, N, bias, relu);
+        // rows with very many slots (the last n_big rows) get a workgroup each; the others
+        // share one between 4, 2 or 1 rows depending on how many threads N can use
+        const int n_split = (int)h->n_split_rows, n_big = (int)h->n_big_rows, n_small = n_split - n_big;
+        const int64_t first = h->rows - h->n_split_rows;
+        if (n_small > 0) {
+            if (N <= 64)
+                long_row_reduce_kernel<4><<<dim3((unsigned)((n_small + 3) / 4)), dim3(kReduceThreads), 0, stream>>>(
+                    h->partial, h->long_slot, h->perm, first, 0, n_small, Y, N, bias, relu);
+            else if (N <= 128)
+                long_row_reduce_kernel<2><<<dim3((unsigned)((n_small + 1) / 2)), dim3(kReduceThreads), 0, stream>>>(
+                    h->partial, h->long_slot, h->perm, first, 0, n_small, Y, N, bias, relu);
+            else
+                long_row_reduce_kernel<1><<<dim3((unsigned)n_small), dim3(kReduceThreads), 0, stream>>>(
+                    h->partial, h->long_slot, h->perm, first, 0, n_small, Y, N, bias, relu);
+        }
+        if (n_big > 0)
+            long_row_reduce_kernel<1><<<dim3((unsigned)n_big), dim3(kReduceThreads), 0, stream>>>(
+                h->partial, h->long_slot, h->perm, first, n_small, n_split, Y, N, bias, relu);
     }
     ACCEL_HIP(hipGetLastError());
     return ACCEL_OK;
