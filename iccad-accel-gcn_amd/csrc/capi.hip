@@ -357,6 +357,18 @@ int accel_set_plan_unit(accel_handle *h, int unit_nz)
     return ACCEL_OK;
 }
 
+int accel_set_plan_groups(accel_handle *h, int groups)
+{
+    clear_error();
+    if (!h) { set_error("accel_set_plan_groups: null handle"); return ACCEL_ERR_ARG; }
+    if (groups != 0 && groups != 8 && groups != 16 && groups != 32 && groups != 64) {
+        set_error("accel_set_plan_groups: groups must be 0 (automatic), 8, 16, 32 or 64, got %d", groups);
+        return ACCEL_ERR_ARG;
+    }
+    h->plan_groups = groups;
+    return ACCEL_OK;
+}
+
 int accel_preprocess(accel_handle *h)
 {
     clear_error();
@@ -380,7 +392,7 @@ int accel_get_info(const accel_handle *h, accel_info *out)
     out->n_plan_units = h->n_units;
     out->n_split_rows = h->n_split_rows;
     out->plan_unit_nz = h->plan_unit;
-    out->reserved = 0;
+    out->plan_groups = h->plan_groups;
     return ACCEL_OK;
 }
 

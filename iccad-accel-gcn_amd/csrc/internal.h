@@ -20,10 +20,32 @@ constexpr int kXcds = 8;                              // accelerator dies, each 
 #endif
 constexpr int kWavesPerGroup = ACCEL_WAVES_PER_GROUP; // wavefronts (work units) per workgroup
 
-// Column group of a non-zero: which die's L2 should hold that row of X.  Eight
-// consecutive columns share a group so that neighbouring short rows of X (one
-// 128-byte line holds 8 rows at N = 4) stay together.
-__host__ __device__ inline int col_group(int c) { return (c >> 3) & (kXcds - 1); }
+constexpr int kMaxGroups = 64;                        // column groups of the launch plan (8..64)
+
+// Column group of a non-zero.  Eight consecutive columns share a group so that
+// neighbouring short rows of X (one 128-byte line holds 8 rows at N = 4) stay
+// together.  Group g belongs to die g % 8; with more than 8 groups a die works
+// through its groups one after the other, so that the share of X its L2 has to
+// hold at any time is 1/groups of the matrix.
+__host__ __device__ inline int col_group(int c, int groups) { return (c >> 3) & (groups - 1); }
+
+// Column groups a split row of degree d is stored in: as many as leave a group about
+// ACCEL_GROUP_MIN_PIECE non-zeros, 8 at least, 64 at most (a power of two); `forced`
+// (8..64) overrides the rule.  Short split rows keep few, long pieces; very long rows
+// are spread over many groups, whose share of X is small enough to stay in one L2.
+#ifndef ACCEL_GROUP_MIN_PIECE
+#define ACCEL_GROUP_MIN_PIECE 96
+#endif
+__host__ __device__ inline int row_groups(int d, int forced)
+{
+    if (forced) return forced;
+    int g = kXcds;
+    while (g < kMaxGroups && d / (2 * g) >= ACCEL_GROUP_MIN_PIECE) g *= 2;
+    return g;
+}
+// Pieces are binned by (groups of their row, group): 8 + 16 + 32 + 64 bins.
+constexpr int kPlanBins = 120;
+__host__ __device__ inline int plan_bin(int groups, int g) { return groups - kXcds + g; }
 
 // last-error string of the calling thread
 void set_error(const char *fmt, ...);
@@ -54,6 +76,7 @@ __host__ __device__ inline void slice_rule(int d, int &w_nz, int &rows_per_block
 
 // The operator state behind the opaque C handle.
 struct accel_handle {
+    static constexpr int kXcds = accel::kXcds;
     int64_t rows = 0, cols = 0, nnz = 0;
     int device = 0;
     // caller's CSR on the device (owned when uploaded from the host)
@@ -80,6 +103,7 @@ struct accel_handle {
     // units of whole rows holding at most plan_unit non-zeros.  384 = one unit per entry.
     int plan_unit_option = 0;         // 0: choose from the size of the matrix
     int plan_unit = ACCEL_DEG_BOUND;
+    int plan_groups = 0;              // 0: by row length (row_groups); 8..64: the same for all rows
     int64_t n_split_rows = 0;         // rows with more than plan_unit non-zeros
     int64_t n_big_rows = 0;           // of those, rows with more than 32 * plan_unit
     int64_t n_blocks = 0, n_long_blocks = 0, n_long_rows = 0, n_zero_rows = 0;

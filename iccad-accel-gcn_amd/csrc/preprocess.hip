@@ -328,26 +328,27 @@ __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
 __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
     const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
     const float *__restrict__ val, const int32_t *__restrict__ perm,
-    const int32_t *__restrict__ s_indptr, int64_t first_long_row, int32_t *__restrict__ s_idx,
-    float *__restrict__ s_val, int *__restrict__ counts)
+    const int32_t *__restrict__ s_indptr, int64_t first_long_row, int forced_groups,
+    int32_t *__restrict__ s_idx, float *__restrict__ s_val, int *__restrict__ counts)
 {
-    __shared__ int cnt[kXcds];
-    __shared__ int base[kXcds];
-    __shared__ int wave_cnt[2][kThreads / 64][kXcds];
+    __shared__ int cnt[kMaxGroups];
+    __shared__ int base[kMaxGroups];
+    __shared__ int wave_cnt[2][kThreads / 64][kMaxGroups];
     const int64_t r = first_long_row + blockIdx.x;
     const int64_t src0 = indptr[perm ? perm[r] : r];
     const int64_t dst0 = s_indptr[r];
     const int d = s_indptr[r + 1] - s_indptr[r];
+    const int ng = row_groups(d, forced_groups);
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    if (threadIdx.x < kXcds) cnt[threadIdx.x] = 0;
+    if ((int)threadIdx.x < kMaxGroups) cnt[threadIdx.x] = 0;
     __syncthreads();
-    for (int i = threadIdx.x; i < d; i += kThreads) atomicAdd(&cnt[col_group(idx[src0 + i])], 1);
+    for (int i = threadIdx.x; i < d; i += kThreads) atomicAdd(&cnt[col_group(idx[src0 + i], ng)], 1);
     __syncthreads();
-    if (threadIdx.x < kXcds) {
+    if ((int)threadIdx.x < kMaxGroups) {              // groups beyond ng stay empty
         int b = 0;
         for (int g = 0; g < (int)threadIdx.x; g++) b += cnt[g];
         base[threadIdx.x] = b;
-        counts[(int64_t)blockIdx.x * kXcds + threadIdx.x] = cnt[threadIdx.x];
+        counts[(int64_t)blockIdx.x * kMaxGroups + threadIdx.x] = cnt[threadIdx.x];
     }
     __syncthreads();
     int flip = 0;
@@ -356,14 +357,18 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
         const bool valid = i < d;
         const int col = valid ? idx[src0 + i] : 0;
         const float v = valid ? val[src0 + i] : 0.0f;
-        const int g = col_group(col);
-        int rank = 0;
+        const int g = col_group(col, ng);
+        wave_cnt[flip][w][lane] = 0;                    // each wavefront clears its own row
+        // lanes of this wavefront with the same group
+        unsigned long long peers = __ballot(valid);
 #pragma unroll
-        for (int gg = 0; gg < kXcds; gg++) {
-            const unsigned long long m = __ballot(valid && g == gg);
-            if (g == gg) rank = __popcll(m & ((1ull << lane) - 1ull));
-            if (lane == 0) wave_cnt[flip][w][gg] = __popcll(m);
+        for (int b = 0; b < 6; b++) {
+            const bool bit = (g >> b) & 1;
+            const unsigned long long bal = __ballot(bit);
+            peers &= bit ? bal : ~bal;
         }
+        const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+        if (valid && rank == 0) wave_cnt[flip][w][g] = __popcll(peers);
         __syncthreads();
         if (valid) {
             int pos = base[g] + rank;
@@ -372,14 +377,14 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
             s_val[dst0 + pos] = v;
         }
         __syncthreads();
-        if (threadIdx.x < kXcds) {
+        if ((int)threadIdx.x < kMaxGroups) {
             int add = 0;
 #pragma unroll
             for (int q = 0; q < kThreads / 64; q++) add += wave_cnt[flip][q][threadIdx.x];
             base[threadIdx.x] += add;
         }
-        // the next round writes the other half of wave_cnt and reads base only
-        // after its own barrier, so no third barrier is needed here
+        // the next round uses the other half of wave_cnt and reads base only after
+        // its own barrier, so no third barrier is needed here
     }
 }
 
@@ -442,7 +447,10 @@ __global__ __launch_bounds__(kThreads) void emit_block4_kernel(
 // ---------------------------------------------------------------------------
 struct PlanParams {
     int queue_long[kXcds];   // long-row units already in each queue
-    int quota[kXcds];        // block4 entries of short rows each queue takes
+    int quota[kXcds];        // units of whole rows each queue takes
+};
+struct BinOffsets {
+    int off[kPlanBins];      // where the pieces of a (row class, column group) bin start in their queue
 };
 
 __device__ __forceinline__ int64_t plan_index(int queue, int pos)
@@ -451,17 +459,19 @@ __device__ __forceinline__ int64_t plan_index(int queue, int pos)
     return ((int64_t)(pos / kWavesPerGroup) * kXcds + queue) * kWavesPerGroup + pos % kWavesPerGroup;
 }
 
+// grp_units is laid out [bin][split row, largest first] and must be zero on entry.
 __global__ __launch_bounds__(kThreads) void long_unit_count_kernel(
-    const int *__restrict__ gcount, int n_long, int piece, int *__restrict__ row_units,
+    const int *__restrict__ gcount, const int32_t *__restrict__ s_indptr, int64_t first_long,
+    int n_long, int forced_groups, int piece, int *__restrict__ row_units,
     int *__restrict__ grp_units)
 {
     const int lr = blockIdx.x * kThreads + threadIdx.x;
     if (lr >= n_long) return;
+    const int ng = row_groups(s_indptr[first_long + lr + 1] - s_indptr[first_long + lr], forced_groups);
     int tot = 0;
-#pragma unroll
-    for (int g = 0; g < kXcds; g++) {
-        const int u = (gcount[(int64_t)lr * kXcds + g] + piece - 1) / piece;
-        grp_units[(int64_t)g * n_long + (n_long - 1 - lr)] = u;   // largest rows first
+    for (int g = 0; g < ng; g++) {
+        const int u = (gcount[(int64_t)lr * kMaxGroups + g] + piece - 1) / piece;
+        grp_units[(int64_t)plan_bin(ng, g) * n_long + (n_long - 1 - lr)] = u;   // largest rows first
         tot += u;
     }
     row_units[lr] = tot;
@@ -469,32 +479,36 @@ __global__ __launch_bounds__(kThreads) void long_unit_count_kernel(
 
 __global__ void plan_totals_kernel(const int *__restrict__ grp_pos, int n_long, int *__restrict__ out)
 {
-    const int g = threadIdx.x;
-    if (g <= kXcds) out[g] = grp_pos[(int64_t)g * n_long];   // g == 8: grand total
+    const int b = threadIdx.x;
+    if (b <= kPlanBins) out[b] = grp_pos[(int64_t)b * n_long];   // b == kPlanBins: grand total
 }
 
 __global__ __launch_bounds__(kThreads) void emit_long_units_kernel(
     const int *__restrict__ gcount, const int32_t *__restrict__ s_indptr, int64_t first_long,
-    const int *__restrict__ slot, const int *__restrict__ grp_pos, int n_long, int piece,
-    int4 *__restrict__ work)
+    const int *__restrict__ slot, const int *__restrict__ grp_pos, int n_long, int forced_groups,
+    int piece, BinOffsets bo, int4 *__restrict__ work)
 {
     const int t = blockIdx.x * kThreads + threadIdx.x;
-    if (t >= n_long * kXcds) return;
-    const int lr = t / kXcds, g = t % kXcds;
-    const int c = gcount[(int64_t)lr * kXcds + g];
+    if (t >= n_long * kMaxGroups) return;
+    const int lr = t / kMaxGroups, g = t % kMaxGroups;
+    const int row = (int)(first_long + lr);
+    const int ng = row_groups(s_indptr[row + 1] - s_indptr[row], forced_groups);
+    if (g >= ng) return;
+    const int c = gcount[(int64_t)lr * kMaxGroups + g];
     if (c == 0) return;
     int c_before = 0, u_before = 0;
     for (int q = 0; q < g; q++) {
-        const int cq = gcount[(int64_t)lr * kXcds + q];
+        const int cq = gcount[(int64_t)lr * kMaxGroups + q];
         c_before += cq;
         u_before += (cq + piece - 1) / piece;
     }
-    const int row = (int)(first_long + lr);
     const int loc = s_indptr[row] + c_before;
-    const int pos0 = grp_pos[(int64_t)g * n_long + (n_long - 1 - lr)] - grp_pos[(int64_t)g * n_long];
+    const int bin = plan_bin(ng, g);
+    const int pos0 = bo.off[bin] + grp_pos[(int64_t)bin * n_long + (n_long - 1 - lr)] -
+                     grp_pos[(int64_t)bin * n_long];
     const int sl = slot[lr] + u_before;
     for (int k = 0, off = 0; off < c; k++, off += piece)
-        work[plan_index(g, pos0 + k)] =
+        work[plan_index(g % kXcds, pos0 + k)] =
             make_int4(kDegBound + 1 + sl + k, row, loc + off, min(piece, c - off));
 }
 
@@ -659,26 +673,29 @@ static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_
     // "long" here = rows cut into pieces (more than plan_unit non-zeros); n_short = block4
     // entries of all other rows (they precede the rest in block4)
     const int64_t n_long = h->n_split_rows;
-    const int unit_nz = h->plan_unit;
+    const int unit_nz = h->plan_unit, forced = h->plan_groups;
     DevBuf row_units, grp_units, sums, totals, dslot, scnt;
     int rc;
-    int tot[kXcds + 1] = {0};
+    int tot[kPlanBins + 1] = {0};
     if ((rc = dslot.alloc(sizeof(int) * (size_t)(n_long + 1)))) return rc;
     if (n_long > 0) {
         if ((rc = row_units.alloc(sizeof(int) * (size_t)n_long))) return rc;
-        if ((rc = grp_units.alloc(sizeof(int) * (size_t)(n_long * kXcds + 1)))) return rc;
-        if ((rc = sums.alloc(sizeof(int) * (size_t)(n_long * kXcds / kTile + 4)))) return rc;
-        if ((rc = totals.alloc(sizeof(int) * (kXcds + 1)))) return rc;
+        const int64_t n_bins = (int64_t)kPlanBins * n_long;
+        if ((rc = grp_units.alloc(sizeof(int) * (size_t)(n_bins + 1)))) return rc;
+        if ((rc = sums.alloc(sizeof(int) * (size_t)(n_bins / kTile + 4)))) return rc;
+        if ((rc = totals.alloc(sizeof(int) * (kPlanBins + 1)))) return rc;
+        if ((rc = fill_u32(grp_units.p, 0u, (size_t)n_bins + 1, s))) return rc;
         long_unit_count_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(
-            gcount, (int)n_long, unit_nz, row_units.as<int>(), grp_units.as<int>());
+            gcount, s_indptr, first_long, (int)n_long, forced, unit_nz, row_units.as<int>(),
+            grp_units.as<int>());
         if ((rc = device_scan<SumOp, false>(row_units.as<int>(), n_long, dslot.as<int>(),
                                             dslot.as<int>() + n_long, sums.as<int>(), s)))
             return rc;
-        if ((rc = device_scan<SumOp, false>(grp_units.as<int>(), n_long * kXcds, grp_units.as<int>(),
-                                            grp_units.as<int>() + n_long * kXcds, sums.as<int>(), s)))
+        if ((rc = device_scan<SumOp, false>(grp_units.as<int>(), n_bins, grp_units.as<int>(),
+                                            grp_units.as<int>() + n_bins, sums.as<int>(), s)))
             return rc;
-        plan_totals_kernel<<<dim3(1), dim3(64), 0, s>>>(grp_units.as<int>(), (int)n_long,
-                                                      totals.as<int>());
+        plan_totals_kernel<<<dim3(1), dim3(128), 0, s>>>(grp_units.as<int>(), (int)n_long,
+                                                       totals.as<int>());
         ACCEL_HIP(hipMemcpyAsync(tot, totals.p, sizeof(tot), hipMemcpyDeviceToHost, s));
     } else {
         ACCEL_HIP(hipMemsetAsync(dslot.p, 0, sizeof(int), s));
@@ -702,12 +719,21 @@ static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_
     }
     const int64_t n_short_units = n_short_units32;
     PlanParams pp;
+    BinOffsets bo;
     int64_t longest = 0;
-    for (int g = 0; g < kXcds; g++) {
-        pp.queue_long[g] = tot[g + 1] - tot[g];
-        longest = std::max<int64_t>(longest, pp.queue_long[g]);
-    }
-    const int64_t n_long_units = tot[kXcds];
+    for (int q = 0; q < kXcds; q++) pp.queue_long[q] = 0;
+    for (int b = 0; b < kPlanBins; b++) bo.off[b] = 0;
+    if (n_long > 0)
+        // a die first takes the pieces of the rows with the most groups (the longest
+        // rows), one group after the other, then those of the next class, ...
+        for (int ng = kMaxGroups; ng >= kXcds; ng /= 2)
+            for (int g = 0; g < ng; g++) {
+                const int b = plan_bin(ng, g);
+                bo.off[b] = pp.queue_long[g % kXcds];
+                pp.queue_long[g % kXcds] += tot[b + 1] - tot[b];
+            }
+    for (int q = 0; q < kXcds; q++) longest = std::max<int64_t>(longest, pp.queue_long[q]);
+    const int64_t n_long_units = n_long > 0 ? tot[kPlanBins] : 0;
     const int64_t total = n_long_units + n_short_units;
     int64_t per_queue = std::max(longest, (total + kXcds - 1) / kXcds);
     per_queue = (per_queue + kWavesPerGroup - 1) / kWavesPerGroup * kWavesPerGroup;
@@ -742,9 +768,9 @@ static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_
     if ((rc = dwork.alloc(sizeof(int4) * (size_t)n_units))) return rc;
     if (n_units > 0 && (rc = fill_u32(dwork.p, 0u, (size_t)n_units * 4, s))) return rc;
     if (n_long > 0)
-        emit_long_units_kernel<<<dim3(grid_for(n_long * kXcds)), dim3(kThreads), 0, s>>>(
-            gcount, s_indptr, first_long, dslot.as<int>(), grp_units.as<int>(), (int)n_long, unit_nz,
-            dwork.as<int4>());
+        emit_long_units_kernel<<<dim3(grid_for(n_long * kMaxGroups)), dim3(kThreads), 0, s>>>(
+            gcount, s_indptr, first_long, dslot.as<int>(), grp_units.as<int>(), (int)n_long, forced,
+            unit_nz, bo, dwork.as<int4>());
     if (n_short > 0)
         emit_short_units_kernel<<<dim3(grid_for(n_short)), dim3(kThreads), 0, s>>>(
             reinterpret_cast<const int4 *>(h->block4), (int)n_short, unit_nz, scnt.as<int>(), pp,
@@ -897,10 +923,10 @@ int preprocess_device(accel_handle *h)
                                      hipMemcpyDeviceToDevice, s));
         }
         if (n_long > 0) {
-            if ((rc = gcount.alloc(sizeof(int) * (size_t)n_long * kXcds))) return rc;
+            if ((rc = gcount.alloc(sizeof(int) * (size_t)n_long * kMaxGroups))) return rc;
             group_long_rows_kernel<<<dim3((unsigned)n_long), dim3(kThreads), 0, s>>>(
-                h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), first_long, sidx.as<int32_t>(),
-                sval.as<float>(), gcount.as<int>());
+                h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), first_long, h->plan_groups,
+                sidx.as<int32_t>(), sval.as<float>(), gcount.as<int>());
         }
         ACCEL_HIP(hipGetLastError());
     }
@@ -914,7 +940,7 @@ int preprocess_device(accel_handle *h)
     ACCEL_HIP(hipStreamSynchronize(s));
     h->block4 = b4;
     h->n_blocks = nb;
-    if (nb + (int64_t)kXcds * (n_long + kWavesPerGroup) > (int64_t)INT_MAX) {
+    if (nb + (int64_t)kMaxGroups * n_long + kXcds * kWavesPerGroup > (int64_t)INT_MAX) {
         set_error("the launch plan would exceed 2^31 work units (%lld block4 entries)", (long long)nb);
         return ACCEL_ERR_ARG;
     }

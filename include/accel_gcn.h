@@ -113,6 +113,12 @@ int accel_preprocess(accel_handle *h);
  * of shorter rows are cut into units of whole rows.  The block4 metadata itself
  * never changes.  Call before accel_preprocess. */
 int accel_set_plan_unit(accel_handle *h, int unit_nz);
+/* Number of column groups the pieces of split rows are sorted into: 8, 16, 32 or
+ * 64 for every row, or 0 (the default) to choose per row: 8 groups, doubled while
+ * a group would still get about 96 non-zeros of the row, up to 64.  Group g =
+ * (column >> 3) & (groups - 1) is worked on by die g % 8, one group after the
+ * other.  Call before accel_preprocess. */
+int accel_set_plan_groups(accel_handle *h, int groups);
 
 /* Check externally produced metadata (a .block4 file) against what
  * accel_preprocess built for this CSR; ACCEL_ERR_META if any int differs. */
@@ -130,7 +136,7 @@ typedef struct accel_info {
     int64_t n_plan_units;   /* wavefronts of one launch (launch plan, incl. padding) */
     int64_t n_split_rows;   /* rows cut into pieces that go through partial sums */
     int32_t plan_unit_nz;   /* most non-zeros one wavefront takes (<= 384) */
-    int32_t reserved;
+    int32_t plan_groups;    /* 0: column groups chosen per row from its length; 8..64: forced */
 } accel_info;
 int accel_get_info(const accel_handle *h, accel_info *out);
 
@@ -146,7 +152,8 @@ int accel_get_sorted_csr(const accel_handle *h, int32_t *indptr, int32_t *idx, f
  * whole rows, verbatim.  x > 384: a piece of a long row: partial-sum slot
  * x - 385, sorted row y, first non-zero z, length w <= 384.  w == 0: padding.
  * Workgroup i runs on die i % 8, so units 4*i .. 4*i+3 belong to queue i % 8;
- * the pieces of long rows in queue g only hold columns c with (c >> 3) & 7 == g.
+ * the pieces of split rows in queue g only hold columns c with (c >> 3) & 7 == g,
+ * ordered by column group ((c >> 3) & (groups - 1)) when there are more than 8.
  * Writes up to cap_units quadruples to out (may be NULL) and the count to *n_units. */
 int accel_get_plan(const accel_handle *h, int32_t *out, int64_t cap_units, int64_t *n_units);
 

@@ -204,25 +204,41 @@ def permute_csr(indptr, indices, values, perm):
 N_COLUMN_GROUPS = 8
 
 
-def column_group(col):
-    """Which of the 8 column groups a column belongs to (groups of 8 consecutive
-    columns, round-robin).  This is the build's own layout rule for rows with
-    more than 384 non-zeros; upstream has no counterpart (it never reorders the
-    non-zeros of a row), so it is pinned by its definition and by the SpMM
-    result being unchanged."""
-    return (np.asarray(col) >> 3) & (N_COLUMN_GROUPS - 1)
+def column_group(col, groups=N_COLUMN_GROUPS):
+    """Which column group a column belongs to (groups of 8 consecutive columns,
+    round-robin over ``groups`` = 8, 16, 32 or 64).  This is the build's own
+    layout rule for the rows it cuts into pieces; upstream has no counterpart
+    (it never reorders the non-zeros of a row), so it is pinned by its
+    definition and by the SpMM result being unchanged."""
+    return (np.asarray(col) >> 3) & (groups - 1)
 
 
-def group_long_rows(indptr, indices, values, threshold=DEG_BOUND):
+GROUP_MIN_PIECE = 96
+
+
+def row_groups(d, forced=0):
+    """Column groups a split row of degree d is stored in: 8, doubled while a group
+    would still get about 96 of the row's non-zeros, at most 64; ``forced``
+    (8..64) overrides.  Definition of this build (no upstream counterpart)."""
+    if forced:
+        return forced
+    g = N_COLUMN_GROUPS
+    while g < 64 and d // (2 * g) >= GROUP_MIN_PIECE:
+        g *= 2
+    return g
+
+
+def group_long_rows(indptr, indices, values, threshold=DEG_BOUND, groups=0):
     """Stable partition of the non-zeros of every row with degree > threshold
     (the launch plan's unit size, 384 unless the plan uses smaller units) by
-    column_group(); all other rows are left as they are."""
+    column_group() into row_groups() groups (``groups`` = 0: chosen per row);
+    all other rows are left as they are."""
     indptr = np.asarray(indptr, dtype=np.int64)
     indices = np.array(indices, copy=True)
     values = None if values is None else np.array(values, copy=True)
     for r in np.flatnonzero(np.diff(indptr) > threshold):
         a, b = indptr[r], indptr[r + 1]
-        order = np.argsort(column_group(indices[a:b]), kind="stable")
+        order = np.argsort(column_group(indices[a:b], row_groups(int(b - a), groups)), kind="stable")
         indices[a:b] = indices[a:b][order]
         if values is not None:
             values[a:b] = values[a:b][order]

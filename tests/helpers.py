@@ -36,10 +36,10 @@ def graph_from_degrees(deg, n_cols=None, seed=0, value_mode="uniform"):
     return pkg.synthetic.random_csr(deg.size, n_cols, deg, seed=seed, value_mode=value_mode)
 
 
-def expected_preprocess(indptr, indices, values, unit=384):
+def expected_preprocess(indptr, indices, values, unit=384, groups=0):
     """(perm, sorted indptr/indices/values, block4) from the CPU oracle; ``unit`` is
     the launch plan's unit size (rows above it are stored grouped by column group)."""
     perm = po.degree_sort(indptr)
     sip, six, sval = po.permute_csr(indptr, indices, values, perm)
-    six, sval = po.group_long_rows(sip, six, sval, unit)
+    six, sval = po.group_long_rows(sip, six, sval, unit, groups)
     return perm, sip, six, sval, po.partition_closed_form(sip)

@@ -46,12 +46,13 @@ def test_stage_on_gpu_writes_golden_file(gpu, tmp_path):
         assert (tmp_path / "meta" / f"{name}.block4").read_bytes() == block4_codec.load(name).tobytes()
 
 
-def check_preprocess(gpu, g, plan_unit=None):
-    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_unit)
+def check_preprocess(gpu, g, plan_unit=None, plan_groups=None):
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_unit, plan_groups)
     if plan_unit is not None:
         assert op.info.plan_unit_nz == plan_unit
+    assert op.info.plan_groups == (plan_groups or 0)
     perm, sip, six, sval, b4 = helpers.expected_preprocess(g.indptr, g.indices, g.values,
-                                                           op.info.plan_unit_nz)
+                                                           op.info.plan_unit_nz, op.info.plan_groups)
     assert np.array_equal(op.perm(), perm)
     ip, ix, v = op.sorted_csr()
     assert np.array_equal(ip, sip) and np.array_equal(ix, six) and np.array_equal(v, sval)
@@ -100,7 +101,7 @@ def test_already_sorted_input(gpu, n_long):
     assert np.array_equal(op.perm(), np.arange(g0.n_rows))
     assert np.array_equal(op.block4(), po.partition_closed_form(sip))
     ip, ix, v = op.sorted_csr()
-    gix, gval = po.group_long_rows(sip, six, sval, op.info.plan_unit_nz)
+    gix, gval = po.group_long_rows(sip, six, sval, op.info.plan_unit_nz, op.info.plan_groups)
     assert np.array_equal(ip, sip) and np.array_equal(ix, gix) and np.array_equal(v, gval)
     op.close()
 
@@ -210,9 +211,16 @@ def check_plan(op, n_cols):
     assert np.all(covered == 1)
     # queue of unit e is (e // 4) % 8
     queue = (np.arange(plan.shape[0]) // 4) % 8
+    last = {}
     for e in np.flatnonzero((plan[:, 3] != 0) & (plan[:, 0] > 384)):
         x, y, z, w = plan[e]
-        assert np.all(po.column_group(six[z:z + w]) == queue[e])
+        groups = po.row_groups(int(deg[y]), op.info.plan_groups)
+        fine = po.column_group(six[z:z + w], groups)
+        assert np.all(fine == fine[0]) and fine[0] % 8 == queue[e]   # one group, on its die
+        # a die takes the rows with the most groups first, and its groups in turn
+        key = (-groups, int(fine[0]))
+        assert key >= last.get(queue[e], (-65, 0))
+        last[queue[e]] = key
     # partial-sum slots: 0 .. n-1, each once, contiguous per row in row order
     slots = long_[:, 0] - 385
     assert sorted(slots.tolist()) == list(range(len(long_)))
@@ -238,6 +246,23 @@ def test_launch_plan_hub_graph(gpu):
     op.close()
 
 
+@pytest.mark.parametrize("groups", [8, 16, 32, 64])
+def test_plan_column_groups(gpu, groups):
+    from oracle import spmm_oracle as so
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=8, n_long=12), n_cols=9000, seed=8)
+    assert po.row_groups(385) == 8 and po.row_groups(1535) == 8 and po.row_groups(1536) == 16
+    assert po.row_groups(3072) == 32 and po.row_groups(6144) == 64 and po.row_groups(10 ** 6) == 64
+    op = check_preprocess(gpu, g, plan_groups=groups)
+    check_plan(op, g.n_cols)
+    X = np.random.default_rng(groups).uniform(-1, 1, (g.n_cols, 48)).astype(np.float32)
+    Y = op.matmul(X)
+    assert so.check(Y, g.indptr, g.indices, g.values, X) <= so.TOL
+    op.close()
+    with pytest.raises(gpu.AccelError) as e:
+        gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_groups=12)
+    assert e.value.status == gpu._lib.ERR_ARG
+
+
 @pytest.mark.parametrize("unit", [16, 50, 96, 200, 384])
 def test_plan_unit_sizes(gpu, unit):
     """Smaller units change the plan and which rows are stored grouped, never the
@@ -255,3 +280,17 @@ def test_plan_unit_sizes(gpu, unit):
     with pytest.raises(gpu.AccelError) as e:
         gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_unit=1000)
     assert e.value.status == gpu._lib.ERR_ARG
+
+
+def test_plan_groups_follow_row_length(gpu):
+    """Automatic rule: rows of 385..1535 non-zeros use 8 column groups, longer rows
+    16, 32 or 64; the plan serves the rows with the most groups first."""
+    from oracle import spmm_oracle as so
+    deg = np.array([5, 400, 1500, 1600, 3100, 6200, 12500, 20000, 1, 0, 64, 3000], dtype=np.int64)
+    g = helpers.graph_from_degrees(deg, n_cols=30_000, seed=3)
+    op = check_preprocess(gpu, g)
+    assert op.info.plan_groups == 0
+    check_plan(op, g.n_cols)
+    X = np.random.default_rng(3).standard_normal((g.n_cols, 32)).astype(np.float32)
+    assert so.check(op.matmul(X), g.indptr, g.indices, g.values, X) <= so.TOL
+    op.close()
