@@ -357,6 +357,18 @@ int accel_set_plan_unit(accel_handle *h, int unit_nz)
     return ACCEL_OK;
 }
 
+int accel_set_plan_split(accel_handle *h, int split_nz)
+{
+    clear_error();
+    if (!h) { set_error("accel_set_plan_split: null handle"); return ACCEL_ERR_ARG; }
+    if (split_nz != 0 && (split_nz < 16 || split_nz > kDegBound)) {
+        set_error("accel_set_plan_split: threshold must be 0 (automatic) or 16..384, got %d", split_nz);
+        return ACCEL_ERR_ARG;
+    }
+    h->plan_split_option = split_nz;
+    return ACCEL_OK;
+}
+
 int accel_set_plan_groups(accel_handle *h, int groups)
 {
     clear_error();
@@ -393,6 +405,8 @@ int accel_get_info(const accel_handle *h, accel_info *out)
     out->n_split_rows = h->n_split_rows;
     out->plan_unit_nz = h->plan_unit;
     out->plan_groups = h->plan_groups;
+    out->plan_split_nz = h->plan_split;
+    out->reserved = 0;
     return ACCEL_OK;
 }
 

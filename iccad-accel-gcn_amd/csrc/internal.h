@@ -98,14 +98,16 @@ struct accel_handle {
     int64_t n_units = 0;              // multiple of 4 * kXcds
     int64_t n_long_units = 0;         // units that write a partial sum
     int32_t *long_slot = nullptr;     // [n_split_rows+1] partial-sum slots of each split row
-    // plan granularity: rows with more than plan_unit non-zeros are cut into pieces of at
+    // plan granularity: rows with more than plan_split non-zeros are cut into pieces of at
     // most plan_unit (through partial sums); block4 entries of shorter rows are cut into
     // units of whole rows holding at most plan_unit non-zeros.  384 = one unit per entry.
     int plan_unit_option = 0;         // 0: choose from the size of the matrix
     int plan_unit = ACCEL_DEG_BOUND;
+    int plan_split_option = 0;        // 0: choose
+    int plan_split = ACCEL_DEG_BOUND; // rows with more non-zeros than this are cut into pieces (<= plan_unit)
     int plan_groups = 0;              // 0: by row length (row_groups); 8..64: the same for all rows
-    int64_t n_split_rows = 0;         // rows with more than plan_unit non-zeros
-    int64_t n_big_rows = 0;           // of those, rows with more than 32 * plan_unit
+    int64_t n_split_rows = 0;         // rows with more than plan_split non-zeros
+    int64_t n_big_rows = 0;           // of those, rows with more than 32 * plan_split
     int64_t n_blocks = 0, n_long_blocks = 0, n_long_rows = 0, n_zero_rows = 0;
     int32_t max_degree = 0;
     double preprocess_ms = 0.0;

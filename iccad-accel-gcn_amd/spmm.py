@@ -59,14 +59,18 @@ class AccelSpMM:
         self._info = None
 
     # -- preprocess ---------------------------------------------------------
-    def preprocess(self, plan_unit: int | None = None, plan_groups: int | None = None) -> "AccelSpMM":
+    def preprocess(self, plan_unit: int | None = None, plan_groups: int | None = None,
+                   plan_split: int | None = None) -> "AccelSpMM":
         """Degree sort, block4 metadata and launch plan on the GPU.  ``plan_unit``
         (16..384) overrides the automatic choice of non-zeros per wavefront,
-        ``plan_groups`` (8, 16, 32, 64) that of column groups for split rows."""
+        ``plan_groups`` (8, 16, 32, 64) that of column groups for split rows,
+        ``plan_split`` (16..384) the row length above which rows are split."""
         if plan_unit is not None:
             check(lib().accel_set_plan_unit(self._h, int(plan_unit)))
         if plan_groups is not None:
             check(lib().accel_set_plan_groups(self._h, int(plan_groups)))
+        if plan_split is not None:
+            check(lib().accel_set_plan_split(self._h, int(plan_split)))
         check(lib().accel_preprocess(self._h))
         info = Info()
         check(lib().accel_get_info(self._h, C.byref(info)))

@@ -108,11 +108,15 @@ int accel_preprocess(accel_handle *h);
 
 /* Granularity of the launch plan (no counterpart upstream, whose unit is always one
  * block4 entry): the most non-zeros one wavefront takes, 16..384, or 0 to let the
- * library choose from the size of the matrix (the default).  Rows with more
- * non-zeros are cut into pieces added up through partial sums; block4 entries
- * of shorter rows are cut into units of whole rows.  The block4 metadata itself
+ * library choose from the size of the matrix (the default).  Rows above the split
+ * threshold (see accel_set_plan_split) are cut into pieces of at most this size,
+ * added up through partial sums; block4 entries of shorter rows are cut into
+ * units of whole rows of at most this size.  The block4 metadata itself
  * never changes.  Call before accel_preprocess. */
 int accel_set_plan_unit(accel_handle *h, int unit_nz);
+/* Rows with more non-zeros than this (16..384, never above the unit size; 0 = let
+ * the library choose) are the ones stored by column group and cut into pieces. */
+int accel_set_plan_split(accel_handle *h, int split_nz);
 /* Number of column groups the pieces of split rows are sorted into: 8, 16, 32 or
  * 64 for every row, or 0 (the default) to choose per row: 8 groups, doubled while
  * a group would still get about 96 non-zeros of the row, up to 64.  Group g =
@@ -137,6 +141,8 @@ typedef struct accel_info {
     int64_t n_split_rows;   /* rows cut into pieces that go through partial sums */
     int32_t plan_unit_nz;   /* most non-zeros one wavefront takes (<= 384) */
     int32_t plan_groups;    /* 0: column groups chosen per row from its length; 8..64: forced */
+    int32_t plan_split_nz;  /* rows with more non-zeros than this are cut into pieces */
+    int32_t reserved;
 } accel_info;
 int accel_get_info(const accel_handle *h, accel_info *out);
 

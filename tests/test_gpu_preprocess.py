@@ -46,13 +46,15 @@ def test_stage_on_gpu_writes_golden_file(gpu, tmp_path):
         assert (tmp_path / "meta" / f"{name}.block4").read_bytes() == block4_codec.load(name).tobytes()
 
 
-def check_preprocess(gpu, g, plan_unit=None, plan_groups=None):
-    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_unit, plan_groups)
+def check_preprocess(gpu, g, plan_unit=None, plan_groups=None, plan_split=None):
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_unit, plan_groups, plan_split)
+    if plan_split is not None:
+        assert op.info.plan_split_nz == min(plan_split, op.info.plan_unit_nz)
     if plan_unit is not None:
         assert op.info.plan_unit_nz == plan_unit
     assert op.info.plan_groups == (plan_groups or 0)
     perm, sip, six, sval, b4 = helpers.expected_preprocess(g.indptr, g.indices, g.values,
-                                                           op.info.plan_unit_nz, op.info.plan_groups)
+                                                           op.info.plan_split_nz, op.info.plan_groups)
     assert np.array_equal(op.perm(), perm)
     ip, ix, v = op.sorted_csr()
     assert np.array_equal(ip, sip) and np.array_equal(ix, six) and np.array_equal(v, sval)
@@ -64,7 +66,7 @@ def check_preprocess(gpu, g, plan_unit=None, plan_groups=None):
     assert info.n_zero_rows == int((d == 0).sum()) and info.n_long_rows == int((d > 384).sum())
     assert info.n_long_blocks == int(np.sum(-(-d[d > 384] // 384)))
     assert info.max_degree == int(d.max(initial=0))
-    assert info.n_split_rows == int((d > info.plan_unit_nz).sum())
+    assert info.n_split_rows == int((d > info.plan_split_nz).sum())
     op.check_block4(b4)
     return op
 
@@ -101,7 +103,7 @@ def test_already_sorted_input(gpu, n_long):
     assert np.array_equal(op.perm(), np.arange(g0.n_rows))
     assert np.array_equal(op.block4(), po.partition_closed_form(sip))
     ip, ix, v = op.sorted_csr()
-    gix, gval = po.group_long_rows(sip, six, sval, op.info.plan_unit_nz, op.info.plan_groups)
+    gix, gval = po.group_long_rows(sip, six, sval, op.info.plan_split_nz, op.info.plan_groups)
     assert np.array_equal(ip, sip) and np.array_equal(ix, gix) and np.array_equal(v, gval)
     op.close()
 
@@ -182,7 +184,7 @@ def check_plan(op, n_cols):
     inside one block4 entry and hold at most plan_unit non-zeros (or one row); pieces of
     split rows hold at most plan_unit non-zeros of one column group and are queued on the
     die that owns that group."""
-    unit = op.info.plan_unit_nz
+    unit, split = op.info.plan_unit_nz, op.info.plan_split_nz
     plan = op.plan().astype(np.int64)
     b4 = op.block4().astype(np.int64)
     sip, six, _ = op.sorted_csr()
@@ -194,7 +196,7 @@ def check_plan(op, n_cols):
     covered = np.zeros(six.size, dtype=np.int32)
     for x, y, z, w in long_:
         covered[z:z + w] += 1
-        assert 0 < w <= unit and sip[y] <= z and z + w <= sip[y + 1] and deg[y] > unit
+        assert 0 < w <= unit and sip[y] <= z and z + w <= sip[y + 1] and deg[y] > split
     entry_of_row = {}
     for d, r, loc, info in b4[b4[:, 0] <= 384]:
         for q in range(info & 0xFFFF):
@@ -202,12 +204,12 @@ def check_plan(op, n_cols):
     for d, r, loc, info in short:
         n = info & 0xFFFF
         covered[loc:loc + d * n] += 1
-        assert d <= unit and (n * d <= unit or n == 1)
+        assert d <= split and (n * d <= unit or n == 1)
         ed, er, eloc, ew = entry_of_row[r]                       # same block4 entry, same fields
         assert ed == d and loc == sip[r] and (info >> 16) == ew
         assert entry_of_row[r + n - 1][1] == er
     if unit == 384:
-        assert sorted(map(tuple, short)) == sorted(map(tuple, b4[b4[:, 0] <= 384]))   # entries verbatim
+        assert sorted(map(tuple, short)) == sorted(map(tuple, b4[b4[:, 0] <= split]))   # entries verbatim
     assert np.all(covered == 1)
     # queue of unit e is (e // 4) % 8
     queue = (np.arange(plan.shape[0]) // 4) % 8
@@ -292,5 +294,16 @@ def test_plan_groups_follow_row_length(gpu):
     assert op.info.plan_groups == 0
     check_plan(op, g.n_cols)
     X = np.random.default_rng(3).standard_normal((g.n_cols, 32)).astype(np.float32)
+    assert so.check(op.matmul(X), g.indptr, g.indices, g.values, X) <= so.TOL
+    op.close()
+
+
+@pytest.mark.parametrize("unit,split", [(384, 100), (384, 200), (128, 40), (96, 384)])
+def test_plan_split_threshold(gpu, unit, split):
+    from oracle import spmm_oracle as so
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=9, n_long=6), seed=9)
+    op = check_preprocess(gpu, g, plan_unit=unit, plan_split=split)
+    check_plan(op, g.n_cols)
+    X = np.random.default_rng(split).uniform(-1, 1, (g.n_cols, 40)).astype(np.float32)
     assert so.check(op.matmul(X), g.indptr, g.indices, g.values, X) <= so.TOL
     op.close()
