@@ -320,10 +320,10 @@ __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Long rows (more than 384 non-zeros): the row's non-zeros are written to the
-// sorted CSR grouped by col_group(column), stably inside each group, so that a
-// work unit of such a row touches rows of X that belong to one die's share.
-// One workgroup per long row; counts[lr*8 + g] receives the size of each group.
+// Split rows: the row's non-zeros are written to the sorted CSR grouped by
+// col_group(column, row_groups(degree)), stably inside each group, so that a
+// work unit of such a row touches rows of X that belong to one column group.
+// One workgroup per split row; counts[lr*64 + g] receives the size of each group.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
     const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
@@ -655,18 +655,21 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
 
 // The launch plan.  One work unit per wavefront, kWavesPerGroup units per
 // workgroup, as int4 (x, y, z, w):
-//   x <= 384 : a block4 entry for whole rows, copied verbatim (degree, first
-//              row, first non-zero, (w_nz << 16) + n_rows);
-//   x  > 384 : a piece of a long row: partial-sum slot x - 385, row y, first
-//              non-zero z, length w <= 384, all of one column group;
+//   x <= 384 : whole rows of one block4 entry (degree, first row, first non-zero,
+//              (w_nz << 16) + n_rows): the entry itself, or a run of its rows when
+//              the plan's unit is smaller than the entry;
+//   x  > 384 : a piece of a split row: partial-sum slot x - 385, row y, first
+//              non-zero z, length w <= plan_unit, all of one column group;
 //   w == 0   : padding, nothing to do.
 // Workgroups are dispatched to the eight dies round-robin (workgroup i runs on
-// die i % 8), so the list is laid out as eight interleaved queues: units of
-// column group g of the long rows go to queue g, whose die then keeps that
-// share of X in its own L2; block4 entries of short rows are dealt to the
-// queues in rounds until all queues are equally long.  Every queue runs its
-// heaviest units first.  Only nine integers travel to the host (the queue
-// lengths), to size the list.
+// die i % 8), so the list is laid out as eight interleaved queues.  Column group
+// g belongs to die g % 8.  A queue holds, in this order: the pieces of the rows
+// stored in 64 groups (the longest rows), one group after the other, largest
+// rows first; then the same for the rows with 32, 16 and 8 groups; then the
+// queue's share of the whole-row units, which are dealt to the queues in rounds,
+// highest degree first, until all queues are equally long.  While a die works
+// through one group its L2 only has to hold that group's share of X.  The host
+// sees 121 bin totals and one unit count, to size the queues.
 static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_indptr,
                            int64_t first_long, int64_t n_short, hipStream_t s)
 {
@@ -906,12 +909,12 @@ int preprocess_device(accel_handle *h)
         return rc;
 
     // ---- sorted CSR ---------------------------------------------------------
-    // Rows of degree <= 384 keep their non-zero order; long rows are grouped by
-    // column group.  The caller's arrays are used in place only when the input
-    // was already sorted and has no long row.
-    // rows cut into pieces: the last n_long rows of the sorted order
+    // Split rows (more than plan_split non-zeros: the last n_long rows of the sorted
+    // order) are stored grouped by column group; all other rows keep their non-zero
+    // order.  The caller's arrays are used in place only when the input was already
+    // sorted and has no split row.
     const int64_t n_long = hs.n_split_rows, first_long = rows - n_long;
-    int32_t nnz_short32 = 0;                             // non-zeros of the rows with degree <= 384
+    int32_t nnz_short32 = 0;                             // non-zeros of the rows that are not split
     ACCEL_HIP(hipMemcpyAsync(&nnz_short32, sip.as<int32_t>() + first_long, sizeof(int32_t),
                              hipMemcpyDeviceToHost, s));
     ACCEL_HIP(hipStreamSynchronize(s));

@@ -2,12 +2,13 @@
 //
 // Work decomposition.  Upstream gives one CUDA thread block of 12 32-lane warps
 // to each block4 entry (spmm_accel.cu:18-28).  Here one 64-lane wavefront takes
-// one work unit and a 256-thread workgroup takes four.  A unit is either a
-// block4 entry of whole rows (up to 12 rows of one degree, <= 384 non-zeros in
-// total) or a piece of <= 384 non-zeros of a row with more than 384 non-zeros.
-// The units come from a launch plan built by the preprocessing step; it orders
-// them so that workgroup i, which the hardware places on die i % 8, works on
-// the column group (share of X) that die keeps in its own L2.
+// one work unit and a 256-thread workgroup takes four.  A unit is either whole
+// rows of one block4 entry (up to 12 rows of one degree, <= 384 non-zeros in
+// total) or a piece of <= 384 non-zeros of a split row (every row with more than
+// 384 non-zeros is split; the plan also splits somewhat shorter ones).  The units
+// come from a launch plan built by the preprocessing step; it orders them so that
+// workgroup i, which the hardware places on die i % 8, works on a column group
+// (share of X) that die keeps in its own L2.
 //
 // Inside the wavefront the lanes form G = 64 / L groups of L lanes; a group owns
 // L * VEC consecutive columns of X/Y (VEC = 4 floats = one 16-byte load per lane
@@ -21,7 +22,7 @@
 //
 // The (column index, value) pairs of the unit are first staged in LDS with
 // coalesced loads, one pair per lane; each group then reads its pairs back with
-// broadcast LDS reads.  Pieces of long rows write their partial sums to a
+// broadcast LDS reads.  Pieces of split rows write their partial sums to a
 // scratch buffer and a second small kernel adds them up in a fixed order, so the
 // result is run-to-run deterministic.  Rows of degree 0 are zero-filled by extra
 // workgroups of the same launch: Y = A X holds after every run with no memset.
