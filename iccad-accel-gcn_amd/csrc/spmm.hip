@@ -53,7 +53,15 @@ __host__ __device__ inline int zero_rows_per_group(int N) { return N >= kZeroFlo
 #ifndef ACCEL_PREDICATED
 #define ACCEL_PREDICATED 1                // 1: one masked batch loop; 0: full batches + scalar tail
 #endif
+#ifndef ACCEL_PANEL
+#define ACCEL_PANEL 64                    // column-panel width for wide operands (0: never split)
+#endif
+#ifndef ACCEL_PANEL_MIN_NNZ
+#define ACCEL_PANEL_MIN_NNZ 4000000       // smaller matrices are not worth several launches
+#endif
 constexpr int kUnroll = ACCEL_UNROLL;
+constexpr int kPanel = ACCEL_PANEL;
+constexpr int64_t kPanelMinNnz = ACCEL_PANEL_MIN_NNZ;
 
 template <class T>
 __device__ __forceinline__ T stream_load(const T *p)
@@ -122,9 +130,11 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     const int4 *__restrict__ work, int n_units,
     const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
     const int32_t *__restrict__ perm, const float *__restrict__ X, float *__restrict__ Y,
-    float *__restrict__ partial, int N, int n_zero_rows, int n_zero_groups,
+    float *__restrict__ partial, int N, int ld, int n_zero_rows, int n_zero_groups,
     const float *__restrict__ bias, int relu)
 {
+    // N columns are computed; rows of X, Y and the partial sums are ld floats apart
+    // (ld > N when the launch covers one column panel of a wider operand)
     constexpr int G = 64 / L;        // lane groups per wavefront
     constexpr int CW = L * VEC;      // columns covered per pass
     __shared__ int2 stage[kWaves][kDegBound];
@@ -144,7 +154,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
                 float t = bias ? bias[c + v] : 0.0f;                // A X is 0 for this row
                 fill[v] = relu ? fmaxf(t, 0.0f) : t;
             }
-            store_out<VEC>(Y + out_row * N + c, fill);
+            store_out<VEC>(Y + out_row * ld + c, fill);
         }
         return;
     }
@@ -234,7 +244,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
                     for (int u = 0; u < kUnroll; u++) {
 #pragma unroll
                         for (int v = 0; v < VEC; v++) x[u][v] = 0.0f;
-                        if (ok[u]) load_vec<VEC>(xcol + (int64_t)p[u].x * N, x[u]);
+                        if (ok[u]) load_vec<VEC>(xcol + (int64_t)p[u].x * ld, x[u]);
                     }
 #pragma unroll
                     for (int u = 0; u < kUnroll; u++) {
@@ -251,7 +261,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 #pragma unroll
                     for (int u = 0; u < kUnroll; u++) p[u] = row_st[o + u * gp];
 #pragma unroll
-                    for (int u = 0; u < kUnroll; u++) load_vec<VEC>(xcol + (int64_t)p[u].x * N, x[u]);
+                    for (int u = 0; u < kUnroll; u++) load_vec<VEC>(xcol + (int64_t)p[u].x * ld, x[u]);
 #pragma unroll
                     for (int u = 0; u < kUnroll; u++) {
                         const float a = __int_as_float(p[u].y);
@@ -262,7 +272,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
                 for (; o < d; o += gp) {
                     const int2 p = row_st[o];
                     float x[VEC];
-                    load_vec<VEC>(xcol + (int64_t)p.x * N, x);
+                    load_vec<VEC>(xcol + (int64_t)p.x * ld, x);
                     const float a = __int_as_float(p.y);
 #pragma unroll
                     for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[v], acc[v]);
@@ -277,7 +287,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
             const int64_t out_row = __shfl(my_out, r < n_rows ? r : 0);
             if (live && k == 0) {
                 if (is_long)
-                    store_vec<VEC>(partial + (int64_t)(deg - (kDegBound + 1)) * N + col, acc);
+                    store_vec<VEC>(partial + (int64_t)(deg - (kDegBound + 1)) * ld + col, acc);
                 else {
                     if (bias) {
 #pragma unroll
@@ -287,7 +297,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 #pragma unroll
                         for (int v = 0; v < VEC; v++) acc[v] = fmaxf(acc[v], 0.0f);
                     }
-                    store_out<VEC>(Y + out_row * N + col, acc);
+                    store_out<VEC>(Y + out_row * ld + col, acc);
                 }
             }
         }
@@ -360,13 +370,13 @@ __global__ __launch_bounds__(256) void copy_u32_kernel(uint32_t *__restrict__ ds
 template <int VEC>
 int launch_for_vec(int L, dim3 grid, hipStream_t s, const int4 *work, int n_units,
                    const int32_t *s_idx, const float *s_val, const int32_t *perm, const float *X,
-                   float *Y, float *partial, int N, int n_zero_rows, int n_zero_groups,
+                   float *Y, float *partial, int N, int ld, int n_zero_rows, int n_zero_groups,
                    const float *bias, int relu)
 {
 #define ACCEL_LAUNCH(LL)                                                                      \
     case LL:                                                                                  \
         spmm_gather_kernel<LL, VEC><<<grid, dim3(kWgThreads), 0, s>>>(                        \
-            work, n_units, s_idx, s_val, perm, X, Y, partial, N, n_zero_rows,                 \
+            work, n_units, s_idx, s_val, perm, X, Y, partial, N, ld, n_zero_rows,             \
             n_zero_groups, bias, relu);                                                                  \
         break;
     switch (L) {
@@ -415,8 +425,6 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     int vec = 1;
     if (N % 4 == 0 && align % 16 == 0) vec = 4;
     else if (N % 2 == 0 && align % 8 == 0) vec = 2;
-    int L = 1;
-    while (L * vec < N && L < 64) L <<= 1;
 
     if (h->n_long_units > 0) {
         const size_t need = (size_t)h->n_long_units * (size_t)N;
@@ -433,30 +441,48 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
             h->partial_floats = need;
         }
     }
+    // Wide operands are computed one column panel at a time (all units for the first
+    // panel, then all units for the next): a panel's slice of X is what the L2s have
+    // to hold, and a narrower slice means more rows of X fit.
+    // Measured (panel 64 against one pass): N = 256 on the hub graph -12 %, N = 128 on the
+    // dense and the power-law 100 M-non-zero graphs -7 % and -4 %; no gain when the
+    // columns have no popularity skew or the rows are very short, and a loss when N is
+    // not a multiple of the panel (N = 100: 64 + 36 leaves lanes idle).
+    int panel = N;
+    if (kPanel > 0 && vec == 4 && N > kPanel && N % kPanel == 0 && h->nnz >= kPanelMinNnz &&
+        h->nnz >= 16 * h->rows)
+        panel = kPanel;
+    const int4 *wk = reinterpret_cast<const int4 *>(h->work);
     const int64_t entry_groups = h->n_units / kWaves;
-    // zero-fill workgroups come first; their count is rounded up to a multiple of the
-    // die count so that entry group i still lands on die i % 8 (surplus ones exit at once)
-    const int zr = zero_rows_per_group(N);
-    int64_t zero_groups = (h->n_zero_rows + zr - 1) / zr;
-    zero_groups = (zero_groups + kXcds - 1) / kXcds * kXcds;
-    const int64_t groups = entry_groups + zero_groups;
-    if (groups > 0x7fffffffLL) {
-        set_error("launch of %lld workgroups exceeds the grid limit", (long long)groups);
-        return ACCEL_ERR_ARG;
-    }
-    int rc = ACCEL_OK;
-    if (groups > 0) {
+    for (int c0 = 0; c0 < N; c0 += panel) {
+        const int n = std::min(panel, N - c0);
+        int L = 1;
+        while (L * vec < n && L < 64) L <<= 1;
+        // zero-fill workgroups come first; their count is rounded up to a multiple of the
+        // die count so that entry group i still lands on die i % 8 (surplus ones exit at once)
+        const int zr = zero_rows_per_group(n);
+        int64_t zero_groups = (h->n_zero_rows + zr - 1) / zr;
+        zero_groups = (zero_groups + kXcds - 1) / kXcds * kXcds;
+        const int64_t groups = entry_groups + zero_groups;
+        if (groups > 0x7fffffffLL) {
+            set_error("launch of %lld workgroups exceeds the grid limit", (long long)groups);
+            return ACCEL_ERR_ARG;
+        }
+        if (groups == 0) break;
         const dim3 grid((unsigned)groups);
-        const int4 *wk = reinterpret_cast<const int4 *>(h->work);
+        const float *Xp = X ? X + c0 : X;
+        float *Yp = Y + c0, *Pp = h->partial ? h->partial + c0 : nullptr;
+        const float *bp = bias ? bias + c0 : nullptr;
+        int rc;
         if (vec == 4)
-            rc = launch_for_vec<4>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)zero_groups, bias, relu);
+            rc = launch_for_vec<4>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
+                                   Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu);
         else if (vec == 2)
-            rc = launch_for_vec<2>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)zero_groups, bias, relu);
+            rc = launch_for_vec<2>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
+                                   Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu);
         else
-            rc = launch_for_vec<1>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                                   X, Y, h->partial, N, (int)h->n_zero_rows, (int)zero_groups, bias, relu);
+            rc = launch_for_vec<1>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
+                                   Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu);
         if (rc) return rc;
     }
     if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));

@@ -312,3 +312,31 @@ def test_random_shapes(gpu):
         err = so.check(Y, g.indptr, g.indices, g.values, X)
         assert err <= TOL, (case, n_rows, n_cols, N, err)
         op.close()
+
+
+def test_column_panels(gpu):
+    """Wide operands on a matrix large enough to be computed in 64-column panels
+    (N = 128, 256) next to widths that are not (N = 100, 192 is, 130 is not)."""
+    g = gpu.synthetic.cfg4(n=200_000, n_edges=4_500_000, max_degree=9_000)
+    assert g.nnz >= 4_000_000 and g.nnz >= 16 * g.n_rows
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    for N in (128, 256, 192, 100, 130):
+        X = np.random.default_rng(N).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+        Y = op.matmul(X)
+        assert np.isfinite(Y).all()
+        R, S = c_oracle.spmm_csr_f64(g.indptr, g.indices, g.values, X)
+        assert so.scaled_error(Y, R, S) <= TOL, N
+    # fused epilogue across panels
+    N = 128
+    X = np.random.default_rng(1).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    b = np.random.default_rng(2).uniform(-0.5, 0.5, N).astype(np.float32)
+    dX, db, dY = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer.from_numpy(b), gpu.DeviceBuffer(g.n_rows * N * 4)
+    op.run_epilogue(dX, dY, N, bias=db, relu=True)
+    op.synchronize()
+    R, S = c_oracle.spmm_csr_f64(g.indptr, g.indices, g.values, X)
+    ref = np.maximum(R + b.astype(np.float64), 0.0)
+    Y = dY.to_numpy(np.float32, (g.n_rows, N)).astype(np.float64)
+    assert np.max(np.abs(Y - ref) / np.maximum(S + np.abs(b), 1e-30)) <= TOL
+    for buf in (dX, db, dY):
+        buf.close()
+    op.close()
