@@ -83,3 +83,18 @@ def test_graph_capture_and_replay(gpu, hip):
     ok(hip.hipGraphDestroy(graph))
     ok(hip.hipStreamDestroy(s))
     dX.close(); dY.close(); op.close()
+
+
+def test_torch_tensors_as_operands(gpu):
+    """torch tensors (data_ptr, torch's current stream) straight into the C ABI, in a
+    process that imports torch first so that one HIP runtime serves both."""
+    import importlib.util
+    import subprocess
+    import sys
+    from pathlib import Path
+    if importlib.util.find_spec("torch") is None:
+        pytest.skip("torch is not installed")
+    case = Path(__file__).resolve().parent / "cases" / "torch_interop.py"
+    r = subprocess.run([sys.executable, str(case)], capture_output=True, text=True, timeout=280)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "RESULT" in r.stdout
