@@ -305,19 +305,21 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 }
 
 // Adds the partial sums of each split row in slot order and writes the row.
-// RPW rows share a 256-thread workgroup (256 / RPW threads each): rows with few
-// slots and few columns do not need a whole workgroup.
-template <int RPW>
+// The first n_shared_groups workgroups take rpw rows each (256 / rpw threads per
+// row): rows with few slots and few columns do not need a whole workgroup.  The
+// remaining workgroups take one row each: the rows with very many slots.
 __global__ __launch_bounds__(kReduceThreads) void long_row_reduce_kernel(
     const float *__restrict__ partial, const int32_t *__restrict__ long_slot,
-    const int32_t *__restrict__ perm, int64_t first_split_row, int lr_begin, int lr_end,
-    float *__restrict__ Y, int N, const float *__restrict__ bias, int relu)
+    const int32_t *__restrict__ perm, int64_t first_split_row, int n_shared_rows, int n_shared_groups,
+    int rpw, int n_rows, float *__restrict__ Y, int N, const float *__restrict__ bias, int relu)
 {
-    constexpr int T = kReduceThreads / RPW;        // threads per row
     __shared__ float red[kReduceThreads];
+    const bool shared_group = (int)blockIdx.x < n_shared_groups;
+    const int T = shared_group ? kReduceThreads / rpw : kReduceThreads;   // threads per row
     const int sub_row = threadIdx.x / T, t = threadIdx.x % T;
-    const int lr = lr_begin + (int)blockIdx.x * RPW + sub_row;
-    const bool row_ok = lr < lr_end;
+    const int lr = shared_group ? (int)blockIdx.x * rpw + sub_row
+                                : n_shared_rows + ((int)blockIdx.x - n_shared_groups);
+    const bool row_ok = lr < (shared_group ? n_shared_rows : n_rows);
     const int first = row_ok ? long_slot[lr] : 0;
     const int nseg = row_ok ? long_slot[lr + 1] - first : 0;
     const float *src = partial + (int64_t)first * N;
@@ -487,24 +489,14 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     }
     if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));
     if (h->n_split_rows > 0) {
-        // rows with very many slots (the last n_big rows) get a workgroup each; the others
-        // share one between 4, 2 or 1 rows depending on how many threads N can use
-        const int n_split = (int)h->n_split_rows, n_big = (int)h->n_big_rows, n_small = n_split - n_big;
-        const int64_t first = h->rows - h->n_split_rows;
-        if (n_small > 0) {
-            if (N <= 64)
-                long_row_reduce_kernel<4><<<dim3((unsigned)((n_small + 3) / 4)), dim3(kReduceThreads), 0, stream>>>(
-                    h->partial, h->long_slot, h->perm, first, 0, n_small, Y, N, bias, relu);
-            else if (N <= 128)
-                long_row_reduce_kernel<2><<<dim3((unsigned)((n_small + 1) / 2)), dim3(kReduceThreads), 0, stream>>>(
-                    h->partial, h->long_slot, h->perm, first, 0, n_small, Y, N, bias, relu);
-            else
-                long_row_reduce_kernel<1><<<dim3((unsigned)n_small), dim3(kReduceThreads), 0, stream>>>(
-                    h->partial, h->long_slot, h->perm, first, 0, n_small, Y, N, bias, relu);
-        }
-        if (n_big > 0)
-            long_row_reduce_kernel<1><<<dim3((unsigned)n_big), dim3(kReduceThreads), 0, stream>>>(
-                h->partial, h->long_slot, h->perm, first, n_small, n_split, Y, N, bias, relu);
+        // one launch: rows with very many slots (the last n_big rows) get a workgroup each, the
+        // others share one between 4, 2 or 1 rows depending on how many threads N can use
+        const int n_split = (int)h->n_split_rows, n_big = (int)h->n_big_rows, n_shared = n_split - n_big;
+        const int rpw = N <= 64 ? 4 : N <= 128 ? 2 : 1;
+        const int shared_groups = (n_shared + rpw - 1) / rpw;
+        long_row_reduce_kernel<<<dim3((unsigned)(shared_groups + n_big)), dim3(kReduceThreads), 0, stream>>>(
+            h->partial, h->long_slot, h->perm, h->rows - h->n_split_rows, n_shared, shared_groups, rpw,
+            n_split, Y, N, bias, relu);
     }
     ACCEL_HIP(hipGetLastError());
     return ACCEL_OK;
