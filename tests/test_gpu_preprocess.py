@@ -307,3 +307,19 @@ def test_plan_split_threshold(gpu, unit, split):
     X = np.random.default_rng(split).uniform(-1, 1, (g.n_cols, 40)).astype(np.float32)
     assert so.check(op.matmul(X), g.indptr, g.indices, g.values, X) <= so.TOL
     op.close()
+
+
+def test_device_plumbing(gpu):
+    import ctypes as C
+    a = np.arange(100_003, dtype=np.uint32)
+    src, dst = gpu.DeviceBuffer.from_numpy(a), gpu.DeviceBuffer(a.nbytes)
+    dst.fill_u32(0xDEADBEEF)
+    assert np.all(dst.to_numpy(np.uint32, a.shape) == 0xDEADBEEF)
+    gpu._lib.check(gpu.lib().accel_dev_copy_u32(C.c_void_p(dst.address), C.c_void_p(src.address), a.size, None))
+    gpu._lib.check(gpu.lib().accel_stream_sync(None))
+    assert np.array_equal(dst.to_numpy(np.uint32, a.shape), a)
+    with pytest.raises(ValueError):
+        dst.to_numpy(np.uint32, (a.size + 1,))
+    src.close()
+    dst.close()
+    dst.close()                                  # closing twice is harmless
