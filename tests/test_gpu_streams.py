@@ -98,3 +98,28 @@ def test_torch_tensors_as_operands(gpu):
     r = subprocess.run([sys.executable, str(case)], capture_output=True, text=True, timeout=280)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     assert "RESULT" in r.stdout
+
+
+def test_no_device_memory_leak(gpu, hip):
+    """Create / preprocess / run / destroy in a loop leaves the free device memory
+    where it was (every buffer the handle owns is released)."""
+    hip.hipMemGetInfo.restype = C.c_int
+    free0, free1, total = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=40, n_long=6), seed=40)
+    X = np.random.default_rng(0).uniform(-1, 1, (g.n_cols, 64)).astype(np.float32)
+
+    def cycle():
+        op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+        op.matmul(X)
+        op.preprocess(plan_unit=64)                      # re-preprocessing replaces the products
+        op.matmul(X)
+        op.close()
+
+    cycle()                                              # first use may grow runtime-internal pools
+    gpu._lib.check(gpu.lib().accel_stream_sync(None))
+    ok(hip.hipMemGetInfo(C.byref(free0), C.byref(total)))
+    for _ in range(20):
+        cycle()
+    gpu._lib.check(gpu.lib().accel_stream_sync(None))
+    ok(hip.hipMemGetInfo(C.byref(free1), C.byref(total)))
+    assert free0.value - free1.value < (8 << 20), f"free memory fell by {free0.value - free1.value} bytes"
