@@ -44,15 +44,6 @@ __host__ __device__ inline int zero_rows_per_group(int N) { return N >= kZeroFlo
 #ifndef ACCEL_UNROLL
 #define ACCEL_UNROLL 4                    // gathers in flight per lane in the main loop
 #endif
-#ifndef ACCEL_NT_STREAM
-#define ACCEL_NT_STREAM 0                 // 1: read-once CSR streams bypass cache retention
-#endif
-#ifndef ACCEL_NT_STORE
-#define ACCEL_NT_STORE 0                  // 1: Y rows are stored with the non-temporal hint
-#endif
-#ifndef ACCEL_PREDICATED
-#define ACCEL_PREDICATED 1                // 1: one masked batch loop; 0: full batches + scalar tail
-#endif
 #ifndef ACCEL_PANEL
 #define ACCEL_PANEL 64                    // column-panel width for wide operands (0: never split)
 #endif
@@ -63,31 +54,9 @@ constexpr int kUnroll = ACCEL_UNROLL;
 constexpr int kPanel = ACCEL_PANEL;
 constexpr int64_t kPanelMinNnz = ACCEL_PANEL_MIN_NNZ;
 
-template <class T>
-__device__ __forceinline__ T stream_load(const T *p)
-{
-#if ACCEL_NT_STREAM
-    return __builtin_nontemporal_load(p);
-#else
-    return *p;
-#endif
-}
-
-#ifndef ACCEL_NT_GATHER
-#define ACCEL_NT_GATHER 0                 // experiment: gathers of X with the non-temporal hint
-#endif
-
 template <int VEC>
 __device__ __forceinline__ void load_vec(const float *__restrict__ p, float (&v)[VEC])
 {
-#if ACCEL_NT_GATHER
-    if constexpr (VEC == 4) {
-        typedef float f4 __attribute__((ext_vector_type(4)));
-        const f4 t = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(p));
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-        return;
-    }
-#endif
     if constexpr (VEC == 4) {
         const float4 t = *reinterpret_cast<const float4 *>(p);
         v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
@@ -109,18 +78,6 @@ __device__ __forceinline__ void store_vec(float *__restrict__ p, const float (&v
     } else {
         *p = v[0];
     }
-}
-
-// Y rows are written once and not read again by this launch.
-template <int VEC>
-__device__ __forceinline__ void store_out(float *__restrict__ p, const float (&v)[VEC])
-{
-#if ACCEL_NT_STORE
-#pragma unroll
-    for (int i = 0; i < VEC; i++) __builtin_nontemporal_store(v[i], p + i);
-#else
-    store_vec<VEC>(p, v);
-#endif
 }
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
@@ -154,7 +111,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
                 float t = bias ? bias[c + v] : 0.0f;                // A X is 0 for this row
                 fill[v] = relu ? fmaxf(t, 0.0f) : t;
             }
-            store_out<VEC>(Y + out_row * ld + c, fill);
+            store_vec<VEC>(Y + out_row * ld + c, fill);
         }
         return;
     }
@@ -186,8 +143,8 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
         for (int j = 0; j < kRounds; j++) {
             const int i = lane + 64 * j;
             if (i < total_nz) {
-                ci[j] = stream_load(s_idx + loc + i);
-                cv[j] = stream_load(s_val + loc + i);
+                ci[j] = s_idx[loc + i];
+                cv[j] = s_val[loc + i];
             }
         }
 #pragma unroll
@@ -227,7 +184,6 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
             if (live) {
                 const int2 *row_st = st + r * d;
                 const float *xcol = X + col;
-#if ACCEL_PREDICATED
                 // every batch issues up to kUnroll gathers; lanes past the end of the
                 // row are masked, so a row costs ceil(d / (gp * kUnroll)) round trips
                 for (int o = k; o < d; o += kUnroll * gp) {
@@ -253,31 +209,6 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
                         for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[u][v], acc[v]);
                     }
                 }
-#else
-                int o = k;
-                for (; o + (kUnroll - 1) * gp < d; o += kUnroll * gp) {
-                    int2 p[kUnroll];
-                    float x[kUnroll][VEC];
-#pragma unroll
-                    for (int u = 0; u < kUnroll; u++) p[u] = row_st[o + u * gp];
-#pragma unroll
-                    for (int u = 0; u < kUnroll; u++) load_vec<VEC>(xcol + (int64_t)p[u].x * ld, x[u]);
-#pragma unroll
-                    for (int u = 0; u < kUnroll; u++) {
-                        const float a = __int_as_float(p[u].y);
-#pragma unroll
-                        for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[u][v], acc[v]);
-                    }
-                }
-                for (; o < d; o += gp) {
-                    const int2 p = row_st[o];
-                    float x[VEC];
-                    load_vec<VEC>(xcol + (int64_t)p.x * ld, x);
-                    const float a = __int_as_float(p.y);
-#pragma unroll
-                    for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[v], acc[v]);
-                }
-#endif
             }
             // add the gp partial sums of each row (all lanes take part)
             for (int m = L; m < (L << lg); m <<= 1) {
@@ -297,7 +228,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 #pragma unroll
                         for (int v = 0; v < VEC; v++) acc[v] = fmaxf(acc[v], 0.0f);
                     }
-                    store_out<VEC>(Y + out_row * ld + col, acc);
+                    store_vec<VEC>(Y + out_row * ld + col, acc);
                 }
             }
         }
