@@ -340,3 +340,23 @@ def test_column_panels(gpu):
     for buf in (dX, db, dY):
         buf.close()
     op.close()
+
+
+def test_non_finite_inputs_stay_in_their_rows(gpu, mixed):
+    """Inf/NaN in a row of X reach exactly the rows of Y that reference it (masked
+    lanes and padding never multiply a stray row of X by zero)."""
+    g, op = mixed
+    N = 48
+    rng = np.random.default_rng(5)
+    X = rng.uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    bad_cols = np.unique(g.indices[rng.integers(0, g.nnz, 6)])
+    X[bad_cols[0::2], 3] = np.inf
+    X[bad_cols[1::2], 7] = np.nan
+    X[0, :] = np.nan                       # row 0 of X is where a careless clamp would read
+    Y = op.matmul(X)
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = so.spmm_scipy32(g.indptr, g.indices, g.values, X)
+    assert np.array_equal(np.isnan(Y), np.isnan(ref))
+    assert np.array_equal(np.isinf(Y), np.isinf(ref))
+    fin = np.isfinite(ref)
+    assert np.max(np.abs(Y[fin] - ref[fin])) <= 1e-4
