@@ -120,6 +120,33 @@ def rocsparse_baseline(pkg, op, g, dX, N, iters=10):
     return out, Yr
 
 
+def neighbor_partition_baseline(pkg, g, dX, N, iters=10):
+    """Neighbour-partition SpMM (the scheme of upstream's second comparison kernel,
+    spmm_gnna.cu) on the same resident operands; comparison only."""
+    import ctypes as C
+    path = os.path.join(os.path.dirname(str(pkg._lib.LIB_PATH)), "libaccelgcn_baselines.so")
+    L = C.CDLL(path)
+    L.baseline_neighbor_partition_last_error.restype = C.c_char_p
+    bufs = [pkg.DeviceBuffer.from_numpy(a) for a in (g.indices, g.values)]
+    dY = pkg.DeviceBuffer(g.n_rows * N * 4)
+    ms = (C.c_float * iters)()
+    pre, n_parts = C.c_float(0), C.c_int64(0)
+    indptr = np.ascontiguousarray(g.indptr, dtype=np.int32)
+    rc = L.baseline_neighbor_partition_spmm(
+        indptr.ctypes.data_as(C.c_void_p), C.c_void_p(bufs[0].address), C.c_void_p(bufs[1].address),
+        C.c_int64(g.n_rows), C.c_int64(g.nnz), C.c_void_p(dX.address), C.c_void_p(dY.address),
+        C.c_int32(N), 0, 3, iters, ms, C.byref(pre), C.byref(n_parts))
+    if rc != 0:
+        out, Yn = {"error": L.baseline_neighbor_partition_last_error().decode()}, None
+    else:
+        out = {"ms": round(float(np.median(list(ms))), 5), "preprocess_ms": round(pre.value, 3),
+               "parts": n_parts.value, "part_size": max(1, g.nnz // max(g.n_rows, 1))}
+        Yn = dY.to_numpy(np.float32, (g.n_rows, N))
+    for b in bufs + [dY]:
+        b.close()
+    return out, Yn
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -132,6 +159,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the scipy baseline and the check")
     ap.add_argument("--compare-rocsparse", action="store_true",
                     help="also time rocSPARSE's CSR SpMM on the same operands (comparison only)")
+    ap.add_argument("--compare-neighbor-partition", action="store_true",
+                    help="also time a neighbour-partition kernel with atomics (the scheme of "
+                         "upstream's spmm_gnna.cu) on the same operands (comparison only)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run the plain copy kernel over this many MiB, --steps times "
                          "(known-size reference for the FETCH_SIZE / WRITE_SIZE counters)")
@@ -239,6 +269,16 @@ def main():
         result["rocsparse"] = {"algorithms": rs, "best_ms": best, "ours_ms": round(ours_ms, 5),
                                "speedup_vs_best": round(best / ours_ms, 3) if best else None,
                                "max_abs_diff_vs_last_alg": float(np.max(np.abs(Ymine - Yr))) if Yr.size else 0.0}
+    if a.compare_neighbor_partition:
+        npb, Yn = neighbor_partition_baseline(pkg, g, dX, N)
+        ours, _ = op.time(dX, dY, N, warmup=3, iters=10, split=False)
+        ours_ms = float(np.median(ours))
+        if Yn is not None:
+            Ymine = dY.to_numpy(np.float32, (g.n_rows, N))
+            npb["ours_ms"] = round(ours_ms, 5)
+            npb["speedup"] = round(npb["ms"] / ours_ms, 3)
+            npb["max_abs_diff"] = float(np.max(np.abs(Ymine - Yn))) if Yn.size else 0.0
+        result["neighbor_partition"] = npb
     if not a.no_cpu:
         base, n_rows, Yc = cpu_baseline(g, X, N)
         result["cpu_baseline"] = base

@@ -72,16 +72,17 @@ def build(verbose: bool = False, extra_flags=(), out: Path | None = None) -> Pat
 
 
 def build_baselines(verbose: bool = False) -> Path:
-    """lib/libaccelgcn_baselines.so: comparison baselines (rocSPARSE SpMM).  Kept in
-    its own library: the product library does not link any sparse library."""
+    """lib/libaccelgcn_baselines.so: comparison baselines (rocSPARSE SpMM and a
+    neighbour-partition kernel).  Kept in its own library: the product library does
+    not link any sparse library and holds no comparison code."""
     out = LIB_DIR / "libaccelgcn_baselines.so"
     cmd = [hipcc(), *compile_flags(), "-shared", str(PKG / "baselines" / "rocsparse_spmm.cpp"),
-           "-o", str(out), "-lrocsparse"]
+           str(PKG / "baselines" / "neighbor_partition_spmm.cpp"), "-o", str(out), "-lrocsparse"]
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
-        raise RuntimeError("hipcc failed for baselines/rocsparse_spmm.cpp:\n" + r.stdout)
+        raise RuntimeError("hipcc failed for baselines/*.cpp:\n" + r.stdout)
     return out
 
 
