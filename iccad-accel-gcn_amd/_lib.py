@@ -40,7 +40,7 @@ class Info(C.Structure):
                 ("n_zero_rows", C.c_int64), ("max_degree", C.c_int32), ("already_sorted", C.c_int32),
                 ("preprocess_ms", C.c_double), ("n_plan_units", C.c_int64), ("n_split_rows", C.c_int64),
                 ("plan_unit_nz", C.c_int32), ("plan_groups", C.c_int32),
-                ("plan_split_nz", C.c_int32), ("reserved", C.c_int32)]
+                ("plan_split_nz", C.c_int32), ("plan_team", C.c_int32)]
 
 
 i32p = C.POINTER(C.c_int32)
@@ -71,6 +71,7 @@ SIGNATURES = {
     "accel_set_plan_unit": (C.c_int, [vp, C.c_int]),
     "accel_set_plan_groups": (C.c_int, [vp, C.c_int]),
     "accel_set_plan_split": (C.c_int, [vp, C.c_int]),
+    "accel_set_plan_team": (C.c_int, [vp, C.c_int]),
     "accel_check_block4": (C.c_int, [vp, i32p, C.c_int64]),
     "accel_get_info": (C.c_int, [vp, C.POINTER(Info)]),
     "accel_get_block4": (C.c_int, [vp, i32p, C.c_int64]),

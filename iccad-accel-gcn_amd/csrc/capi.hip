@@ -381,6 +381,19 @@ int accel_set_plan_groups(accel_handle *h, int groups)
     return ACCEL_OK;
 }
 
+int accel_set_plan_team(accel_handle *h, int mode)
+{
+    clear_error();
+    if (!h) { set_error("accel_set_plan_team: null handle"); return ACCEL_ERR_ARG; }
+    if (mode < 0 || mode > 2) {
+        set_error("accel_set_plan_team: mode must be 0 (automatic), 1 (wavefront units) or 2 "
+                  "(workgroup units), got %d", mode);
+        return ACCEL_ERR_ARG;
+    }
+    h->plan_team_option = mode;
+    return ACCEL_OK;
+}
+
 int accel_preprocess(accel_handle *h)
 {
     clear_error();
@@ -406,7 +419,7 @@ int accel_get_info(const accel_handle *h, accel_info *out)
     out->plan_unit_nz = h->plan_unit;
     out->plan_groups = h->plan_groups;
     out->plan_split_nz = h->plan_split;
-    out->reserved = 0;
+    out->plan_team = h->plan_team ? 1 : 0;
     return ACCEL_OK;
 }
 

@@ -106,6 +106,8 @@ struct accel_handle {
     int plan_split_option = 0;        // 0: choose
     int plan_split = ACCEL_DEG_BOUND; // rows with more non-zeros than this are cut into pieces (<= plan_unit)
     int plan_groups = 0;              // 0: by row length (row_groups); 8..64: the same for all rows
+    int plan_team_option = 0;         // 0: choose from the size of the matrix; 1: wavefront units; 2: workgroup units
+    bool plan_team = false;           // a unit is worked on by a whole workgroup (small matrices)
     int64_t n_split_rows = 0;         // rows with more than plan_split non-zeros
     int64_t n_big_rows = 0;           // of those, rows with more than 32 * plan_split
     int64_t n_blocks = 0, n_long_blocks = 0, n_long_rows = 0, n_zero_rows = 0;

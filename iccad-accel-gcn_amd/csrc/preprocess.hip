@@ -676,7 +676,8 @@ static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_
     // "long" here = rows cut into pieces (more than plan_split non-zeros); n_short = block4
     // entries of all other rows (they precede the rest in block4)
     const int64_t n_long = h->n_split_rows;
-    const int unit_nz = h->plan_unit, forced = h->plan_groups;
+    // pieces of split rows hold up to piece_nz non-zeros, units of several whole rows up to unit_nz
+    const int unit_nz = h->plan_unit, piece_nz = std::max(h->plan_unit, h->plan_split), forced = h->plan_groups;
     DevBuf row_units, grp_units, sums, totals, dslot, scnt;
     int rc;
     int tot[kPlanBins + 1] = {0};
@@ -689,7 +690,7 @@ static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_
         if ((rc = totals.alloc(sizeof(int) * (kPlanBins + 1)))) return rc;
         if ((rc = fill_u32(grp_units.p, 0u, (size_t)n_bins + 1, s))) return rc;
         long_unit_count_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(
-            gcount, s_indptr, first_long, (int)n_long, forced, unit_nz, row_units.as<int>(),
+            gcount, s_indptr, first_long, (int)n_long, forced, piece_nz, row_units.as<int>(),
             grp_units.as<int>());
         if ((rc = device_scan<SumOp, false>(row_units.as<int>(), n_long, dslot.as<int>(),
                                             dslot.as<int>() + n_long, sums.as<int>(), s)))
@@ -773,7 +774,7 @@ static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_
     if (n_long > 0)
         emit_long_units_kernel<<<dim3(grid_for(n_long * kMaxGroups)), dim3(kThreads), 0, s>>>(
             gcount, s_indptr, first_long, dslot.as<int>(), grp_units.as<int>(), (int)n_long, forced,
-            unit_nz, bo, dwork.as<int4>());
+            piece_nz, bo, dwork.as<int4>());
     if (n_short > 0)
         emit_short_units_kernel<<<dim3(grid_for(n_short)), dim3(kThreads), 0, s>>>(
             reinterpret_cast<const int4 *>(h->block4), (int)n_short, unit_nz, scnt.as<int>(), pp,
@@ -787,16 +788,37 @@ static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_
     return ACCEL_OK;
 }
 
-// Unit size of the launch plan.  Large matrices keep the block4 granularity (384
-// non-zeros per wavefront: fewest descriptors and partial sums, and the launch is
-// bandwidth-bound anyway).  Small ones are latency-bound: the time is set by the
-// longest chain of dependent gathers in one wavefront, so units are made smaller.
-// Measured at N = 16 and 64 on matrices of 0.1 M to 27 M non-zeros: from about 1 M
-// non-zeros on, 384 is best or within 2 %; a 99 k-non-zero matrix runs in 11 us with
-// units of 48 against 17 us with 384, a 208 k one in 12 us with 96 against 14 us.
-static int choose_plan_unit(int64_t rows, int64_t nnz)
+// Small matrices are latency-bound: the time of a launch is the longest chain of
+// dependent memory round trips in one wavefront, not the traffic.  For them a unit is
+// given to a whole workgroup (four wavefronts share its rows, or its row's non-zeros),
+// which shortens that chain, and rows of up to 384 non-zeros stay whole, so that most
+// such matrices need no partial sums and no second launch.
+// Measured (everything one call launches, N = 16 / 64 / 128, wavefront units with their
+// best unit size against workgroup units of 96 with whole rows up to 384):
+//   99 k non-zeros, longest row 171:   10.1 / 11.2 / 16.3 us  ->  7.3 /  9.4 / 11.4 us
+//   208 k non-zeros, power law:        11.8 / 12.4 / 19.8 us  ->  7.9 / 10.5 / 12.6 us
+//   1.2 M, 1.6 M and 2.4 M non-zeros:  wavefront units are faster (26 / 53 / 99 us against
+//                                      34 / 55 / 102 us on the 1.2 M one).
+#ifndef ACCEL_TEAM_MAX_NNZ
+#define ACCEL_TEAM_MAX_NNZ (512 * 1024)
+#endif
+static bool choose_plan_team(int64_t rows, int64_t nnz)
 {
     (void)rows;
+    return nnz < (int64_t)ACCEL_TEAM_MAX_NNZ;
+}
+
+// Unit size of the launch plan: the most non-zeros of a unit of several whole rows (and,
+// with wavefront units, of a piece of a split row).  Large matrices keep the block4
+// granularity (384: fewest descriptors and partial sums, and the launch is bandwidth-bound
+// anyway).  Small ones want short chains: workgroup units of 96 non-zeros (48 below 64 k
+// non-zeros: 10.0 against 11.2 us at N = 64 on a 35 k one).  With wavefront units on a
+// small matrix (only when asked for) 48 / 96 are best too: a 99 k-non-zero matrix 11 us
+// with units of 48 against 17 us with 384; from about 1 M non-zeros on 384 is best or within 2 %.
+static int choose_plan_unit(int64_t rows, int64_t nnz, bool team)
+{
+    (void)rows;
+    if (team) return nnz < (int64_t)64 * 1024 ? 48 : 96;
     if (nnz < (int64_t)128 * 1024) return 48;
     if (nnz < (int64_t)512 * 1024) return 96;
     return kDegBound;
@@ -809,11 +831,11 @@ static int choose_plan_unit(int64_t rows, int64_t nnz)
 #ifndef ACCEL_PLAN_SPLIT
 #define ACCEL_PLAN_SPLIT 192
 #endif
-static int choose_plan_split(int64_t rows, int64_t nnz)
+static int choose_plan_split(int64_t rows, int64_t nnz, bool team)
 {
     (void)rows;
     (void)nnz;
-    return ACCEL_PLAN_SPLIT;
+    return team ? kDegBound : ACCEL_PLAN_SPLIT;        // workgroup units: rows up to one unit stay whole
 }
 
 int preprocess_device(accel_handle *h)
@@ -828,9 +850,12 @@ int preprocess_device(accel_handle *h)
     h->max_degree = 0;
     h->n_units = h->n_long_units = 0;
     h->n_split_rows = h->n_big_rows = 0;
-    h->plan_unit = h->plan_unit_option > 0 ? h->plan_unit_option : choose_plan_unit(rows, nnz);
-    h->plan_split = std::min(h->plan_unit, h->plan_split_option > 0 ? h->plan_split_option
-                                                                    : choose_plan_split(rows, nnz));
+    h->plan_team = h->plan_team_option == 2 || (h->plan_team_option == 0 && choose_plan_team(rows, nnz));
+    h->plan_unit = h->plan_unit_option > 0 ? h->plan_unit_option : choose_plan_unit(rows, nnz, h->plan_team);
+    h->plan_split = h->plan_split_option > 0 ? h->plan_split_option : choose_plan_split(rows, nnz, h->plan_team);
+    // a wavefront never takes more than plan_unit non-zeros; a workgroup takes a whole row of
+    // up to plan_split even when units of several rows are kept smaller
+    if (!h->plan_team) h->plan_split = std::min(h->plan_split, h->plan_unit);
     if (rows == 0) {
         h->identity_perm = true;
         h->ready = true;

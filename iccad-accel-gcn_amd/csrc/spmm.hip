@@ -8,7 +8,8 @@
 // 384 non-zeros is split; the plan also splits somewhat shorter ones).  The units
 // come from a launch plan built by the preprocessing step; it orders them so that
 // workgroup i, which the hardware places on die i % 8, works on a column group
-// (share of X) that die keeps in its own L2.
+// (share of X) that die keeps in its own L2.  Small matrices use the same list with
+// one unit per workgroup instead (spmm_team_kernel below).
 //
 // Inside the wavefront the lanes form G = 64 / L groups of L lanes; a group owns
 // L * VEC consecutive columns of X/Y (VEC = 4 floats = one 16-byte load per lane
@@ -50,7 +51,11 @@ __host__ __device__ inline int zero_rows_per_group(int N) { return N >= kZeroFlo
 #ifndef ACCEL_PANEL_MIN_NNZ
 #define ACCEL_PANEL_MIN_NNZ 4000000       // smaller matrices are not worth several launches
 #endif
+#ifndef ACCEL_TEAM_UNROLL
+#define ACCEL_TEAM_UNROLL 4               // the same for the kernel with workgroup units (8: 5-10 % slower)
+#endif
 constexpr int kUnroll = ACCEL_UNROLL;
+constexpr int kTeamUnroll = ACCEL_TEAM_UNROLL;
 constexpr int kPanel = ACCEL_PANEL;
 constexpr int64_t kPanelMinNnz = ACCEL_PANEL_MIN_NNZ;
 
@@ -82,6 +87,30 @@ __device__ __forceinline__ void store_vec(float *__restrict__ p, const float (&v
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// Zero-degree rows are the first n_zero_rows rows of the sorted order; the workgroups at
+// the head of the grid write them (act(bias) with an epilogue).  They come first so that
+// they do not form a tail.
+template <int VEC>
+__device__ __forceinline__ void zero_fill_rows(const int32_t *__restrict__ perm, float *__restrict__ Y,
+                                               int N, int ld, int n_zero_rows,
+                                               const float *__restrict__ bias, int relu)
+{
+    const int rows_here = zero_rows_per_group(N);
+    const int r0 = (int)blockIdx.x * rows_here;
+    const int n = min(rows_here, n_zero_rows - r0) * N;        // floats of this workgroup
+    float fill[VEC];
+    for (int i = (int)threadIdx.x * VEC; i < n; i += kWgThreads * VEC) {
+        const int r = i / N, c = i - r * N;
+        const int64_t out_row = perm ? perm[r0 + r] : r0 + r;
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+            float t = bias ? bias[c + v] : 0.0f;                // A X is 0 for this row
+            fill[v] = relu ? fmaxf(t, 0.0f) : t;
+        }
+        store_vec<VEC>(Y + out_row * ld + c, fill);
+    }
+}
+
 template <int L, int VEC>
 __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     const int4 *__restrict__ work, int n_units,
@@ -97,22 +126,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     __shared__ int2 stage[kWaves][kDegBound];
 
     if ((int)blockIdx.x < n_zero_groups) {
-        // zero-degree rows: they are the first n_zero_rows rows of the sorted order.
-        // These workgroups come first in the grid so that they do not form a tail.
-        const int rows_here = zero_rows_per_group(N);
-        const int r0 = (int)blockIdx.x * rows_here;
-        const int n = min(rows_here, n_zero_rows - r0) * N;        // floats of this workgroup
-        float fill[VEC];
-        for (int i = (int)threadIdx.x * VEC; i < n; i += kWgThreads * VEC) {
-            const int r = i / N, c = i - r * N;
-            const int64_t out_row = perm ? perm[r0 + r] : r0 + r;
-#pragma unroll
-            for (int v = 0; v < VEC; v++) {
-                float t = bias ? bias[c + v] : 0.0f;                // A X is 0 for this row
-                fill[v] = relu ? fmaxf(t, 0.0f) : t;
-            }
-            store_vec<VEC>(Y + out_row * ld + c, fill);
-        }
+        zero_fill_rows<VEC>(perm, Y, N, ld, n_zero_rows, bias, relu);
         return;
     }
 
@@ -235,6 +249,159 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     }
 }
 
+// The same computation with one unit per workgroup: the four wavefronts form 4 * G lane
+// groups that share the unit's rows, or its row's non-zeros.  When a row's groups span
+// several wavefronts their sums meet in LDS.  Used for small matrices, where the time of
+// a launch is the longest chain of dependent gathers in one wavefront: the chain is four
+// times shorter and rows of up to one unit need no partial sums.
+template <int L, int VEC>
+__global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
+    const int4 *__restrict__ work, int n_units,
+    const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
+    const int32_t *__restrict__ perm, const float *__restrict__ X, float *__restrict__ Y,
+    float *__restrict__ partial, int N, int ld, int n_zero_rows, int n_zero_groups,
+    const float *__restrict__ bias, int relu)
+{
+    constexpr int G = 64 / L;        // lane groups per wavefront
+    constexpr int TG = G * kWaves;   // lane groups per workgroup
+    constexpr int CW = L * VEC;      // columns covered per pass
+    __shared__ int2 stage[kDegBound];
+    __shared__ float meet[kWaves][CW];
+
+    if ((int)blockIdx.x < n_zero_groups) {
+        zero_fill_rows<VEC>(perm, Y, N, ld, n_zero_rows, bias, relu);
+        return;
+    }
+    const int lane = threadIdx.x & 63;
+    const int wv = uniform(threadIdx.x >> 6);
+    const int e = (int)blockIdx.x - n_zero_groups;
+    if (e >= n_units) return;
+    const int4 b = work[e];
+    const int deg = uniform(b.x), row0 = uniform(b.y), loc = uniform(b.z), info = uniform(b.w);
+    if (info == 0) return;                              // padding unit (the whole workgroup leaves)
+    const bool is_long = deg > kDegBound;
+    const int n_rows = is_long ? 1 : (info & 0xFFFF);
+    const int d = is_long ? info : deg;
+    const int total_nz = n_rows * d;
+
+    int my_out = row0 + lane;
+    if (!is_long && perm && lane < n_rows) my_out = perm[row0 + lane];
+
+    {   // stage the unit's (column, value) pairs: 256 threads, at most two rounds
+        constexpr int kRounds = (kDegBound + kWgThreads - 1) / kWgThreads;
+        int ci[kRounds];
+        float cv[kRounds];
+#pragma unroll
+        for (int j = 0; j < kRounds; j++) {
+            const int i = (int)threadIdx.x + kWgThreads * j;
+            if (i < total_nz) {
+                ci[j] = s_idx[loc + i];
+                cv[j] = s_val[loc + i];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kRounds; j++) {
+            const int i = (int)threadIdx.x + kWgThreads * j;
+            if (i < total_nz) stage[i] = make_int2(ci[j], __float_as_int(cv[j]));
+        }
+    }
+    __syncthreads();
+
+    // groups per row: power of two that minimises ceil(n_rows / (TG/gp)) * ceil(d / gp)
+    int lg = 0;
+    {
+        int best = 0x7fffffff;
+#pragma unroll
+        for (int q = 0; (1 << q) <= TG; q++) {
+            const int rows_at_once = TG >> q;
+            const int steps = ((n_rows + rows_at_once - 1) / rows_at_once) * ((d + (1 << q) - 1) >> q);
+            if (steps < best) { best = steps; lg = q; }
+        }
+    }
+    const int gp = 1 << lg;
+    const int rows_at_once = TG >> lg;
+    const int g = lane / L, sub = lane % L;
+    const int vg = wv * G + g;           // this lane group among the workgroup's
+    const int k = vg & (gp - 1);         // which of the row's gp groups this is
+    const int rloc = vg >> lg;           // which of the rows in flight
+    const int in_wave = gp < G ? gp : G;             // groups of one row inside a wavefront
+    const int waves_per_row = gp > G ? gp / G : 1;   // > 1: the row's sums meet in LDS
+
+    for (int c0 = 0; c0 < N; c0 += CW) {
+        const int col = c0 + sub * VEC;
+        const bool col_ok = col < N;
+        for (int r_it = 0; r_it < n_rows; r_it += rows_at_once) {
+            const int r = r_it + rloc;
+            const bool live = col_ok && r < n_rows;
+            float acc[VEC];
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[v] = 0.0f;
+            if (live) {
+                const int2 *row_st = stage + r * d;
+                const float *xcol = X + col;
+                for (int o = k; o < d; o += kTeamUnroll * gp) {
+                    int2 p[kTeamUnroll];
+                    float x[kTeamUnroll][VEC];
+                    bool ok[kTeamUnroll];
+#pragma unroll
+                    for (int u = 0; u < kTeamUnroll; u++) {
+                        const int ou = o + u * gp;
+                        ok[u] = ou < d;
+                        p[u] = row_st[ok[u] ? ou : k];
+                    }
+#pragma unroll
+                    for (int u = 0; u < kTeamUnroll; u++) {
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) x[u][v] = 0.0f;
+                        if (ok[u]) load_vec<VEC>(xcol + (int64_t)p[u].x * ld, x[u]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < kTeamUnroll; u++) {
+                        const float a = ok[u] ? __int_as_float(p[u].y) : 0.0f;
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[u][v], acc[v]);
+                    }
+                }
+            }
+            // the row's groups inside this wavefront (all lanes take part)
+            for (int m = L; m < L * in_wave; m <<= 1) {
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[v] += __shfl_xor(acc[v], m);
+            }
+            if (waves_per_row > 1) {                 // workgroup-uniform
+                if (g == 0) {
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) meet[wv][sub * VEC + v] = acc[v];
+                }
+                __syncthreads();
+                if (wv % waves_per_row == 0 && g == 0) {
+                    for (int q = 1; q < waves_per_row; q++) {
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[v] += meet[wv + q][sub * VEC + v];
+                    }
+                }
+                __syncthreads();
+            }
+            const int64_t out_row = __shfl(my_out, r < n_rows ? r : 0);
+            if (live && k == 0) {
+                if (is_long)
+                    store_vec<VEC>(partial + (int64_t)(deg - (kDegBound + 1)) * ld + col, acc);
+                else {
+                    if (bias) {
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[v] += bias[col + v];
+                    }
+                    if (relu) {
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[v] = fmaxf(acc[v], 0.0f);
+                    }
+                    store_vec<VEC>(Y + out_row * ld + col, acc);
+                }
+            }
+        }
+    }
+}
+
 // Adds the partial sums of each split row in slot order and writes the row.
 // The first n_shared_groups workgroups take rpw rows each (256 / rpw threads per
 // row): rows with few slots and few columns do not need a whole workgroup.  The
@@ -301,16 +468,21 @@ __global__ __launch_bounds__(256) void copy_u32_kernel(uint32_t *__restrict__ ds
 }
 
 template <int VEC>
-int launch_for_vec(int L, dim3 grid, hipStream_t s, const int4 *work, int n_units,
+int launch_for_vec(bool team, int L, dim3 grid, hipStream_t s, const int4 *work, int n_units,
                    const int32_t *s_idx, const float *s_val, const int32_t *perm, const float *X,
                    float *Y, float *partial, int N, int ld, int n_zero_rows, int n_zero_groups,
                    const float *bias, int relu)
 {
 #define ACCEL_LAUNCH(LL)                                                                      \
     case LL:                                                                                  \
-        spmm_gather_kernel<LL, VEC><<<grid, dim3(kWgThreads), 0, s>>>(                        \
-            work, n_units, s_idx, s_val, perm, X, Y, partial, N, ld, n_zero_rows,             \
-            n_zero_groups, bias, relu);                                                                  \
+        if (team)                                                                             \
+            spmm_team_kernel<LL, VEC><<<grid, dim3(kWgThreads), 0, s>>>(                      \
+                work, n_units, s_idx, s_val, perm, X, Y, partial, N, ld, n_zero_rows,         \
+                n_zero_groups, bias, relu);                                                   \
+        else                                                                                  \
+            spmm_gather_kernel<LL, VEC><<<grid, dim3(kWgThreads), 0, s>>>(                    \
+                work, n_units, s_idx, s_val, perm, X, Y, partial, N, ld, n_zero_rows,         \
+                n_zero_groups, bias, relu);                                                   \
         break;
     switch (L) {
         ACCEL_LAUNCH(1)
@@ -386,7 +558,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         h->nnz >= 16 * h->rows)
         panel = kPanel;
     const int4 *wk = reinterpret_cast<const int4 *>(h->work);
-    const int64_t entry_groups = h->n_units / kWaves;
+    const int64_t entry_groups = h->plan_team ? h->n_units : h->n_units / kWaves;
     for (int c0 = 0; c0 < N; c0 += panel) {
         const int n = std::min(panel, N - c0);
         int L = 1;
@@ -408,13 +580,13 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         const float *bp = bias ? bias + c0 : nullptr;
         int rc;
         if (vec == 4)
-            rc = launch_for_vec<4>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
+            rc = launch_for_vec<4>(h->plan_team, L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
                                    Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu);
         else if (vec == 2)
-            rc = launch_for_vec<2>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
+            rc = launch_for_vec<2>(h->plan_team, L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
                                    Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu);
         else
-            rc = launch_for_vec<1>(L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
+            rc = launch_for_vec<1>(h->plan_team, L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
                                    Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu);
         if (rc) return rc;
     }

@@ -60,11 +60,15 @@ class AccelSpMM:
 
     # -- preprocess ---------------------------------------------------------
     def preprocess(self, plan_unit: int | None = None, plan_groups: int | None = None,
-                   plan_split: int | None = None) -> "AccelSpMM":
+                   plan_split: int | None = None, plan_team: int | None = None) -> "AccelSpMM":
         """Degree sort, block4 metadata and launch plan on the GPU.  ``plan_unit``
-        (16..384) overrides the automatic choice of non-zeros per wavefront,
+        (16..384) overrides the automatic choice of non-zeros per unit,
         ``plan_groups`` (8, 16, 32, 64) that of column groups for split rows,
-        ``plan_split`` (16..384) the row length above which rows are split."""
+        ``plan_split`` (16..384) the row length above which rows are split,
+        ``plan_team`` (1: one wavefront per unit, 2: one workgroup per unit) who
+        works on a unit."""
+        if plan_team is not None:
+            check(lib().accel_set_plan_team(self._h, int(plan_team)))
         if plan_unit is not None:
             check(lib().accel_set_plan_unit(self._h, int(plan_unit)))
         if plan_groups is not None:

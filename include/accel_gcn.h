@@ -123,6 +123,13 @@ int accel_set_plan_split(accel_handle *h, int split_nz);
  * (column >> 3) & (groups - 1) is worked on by die g % 8, one group after the
  * other.  Call before accel_preprocess. */
 int accel_set_plan_groups(accel_handle *h, int groups);
+/* Who works on one unit of the launch plan: 1 = one wavefront (four units per
+ * workgroup, the layout described at accel_get_plan); 2 = a whole workgroup of four
+ * wavefronts, which share the unit's rows or, for a long row, its non-zeros; 0 (the
+ * default) = the library chooses: workgroup units for small matrices, whose run time
+ * is the longest chain of dependent gathers rather than memory bandwidth.  Call
+ * before accel_preprocess. */
+int accel_set_plan_team(accel_handle *h, int mode);
 
 /* Check externally produced metadata (a .block4 file) against what
  * accel_preprocess built for this CSR; ACCEL_ERR_META if any int differs. */
@@ -142,7 +149,7 @@ typedef struct accel_info {
     int32_t plan_unit_nz;   /* most non-zeros one wavefront takes (<= 384) */
     int32_t plan_groups;    /* 0: column groups chosen per row from its length; 8..64: forced */
     int32_t plan_split_nz;  /* rows with more non-zeros than this are cut into pieces */
-    int32_t reserved;
+    int32_t plan_team;      /* 1: a unit is worked on by a whole workgroup, 0: by one wavefront */
 } accel_info;
 int accel_get_info(const accel_handle *h, accel_info *out);
 
@@ -154,7 +161,8 @@ int accel_get_sorted_csr(const accel_handle *h, int32_t *indptr, int32_t *idx, f
 
 /* The launch plan derived from block4 (no counterpart upstream, where the grid
  * is simply one thread block per block4 entry, spmm_accel.cu:128): one int4
- * (x, y, z, w) per wavefront, four per workgroup.  x <= 384: a block4 entry of
+ * (x, y, z, w) per wavefront, four per workgroup (per workgroup when
+ * accel_info.plan_team is 1; the list has the same form).  x <= 384: a block4 entry of
  * whole rows, verbatim.  x > 384: a piece of a long row: partial-sum slot
  * x - 385, sorted row y, first non-zero z, length w <= 384.  w == 0: padding.
  * Workgroup i runs on die i % 8, so units 4*i .. 4*i+3 belong to queue i % 8;

@@ -46,10 +46,16 @@ def test_stage_on_gpu_writes_golden_file(gpu, tmp_path):
         assert (tmp_path / "meta" / f"{name}.block4").read_bytes() == block4_codec.load(name).tobytes()
 
 
-def check_preprocess(gpu, g, plan_unit=None, plan_groups=None, plan_split=None):
-    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_unit, plan_groups, plan_split)
+def check_preprocess(gpu, g, plan_unit=None, plan_groups=None, plan_split=None, plan_team=None):
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_unit, plan_groups, plan_split,
+                                                                         plan_team)
+    if plan_team is not None:
+        assert op.info.plan_team == (plan_team == 2)
+    else:
+        assert op.info.plan_team == (g.nnz < 512 * 1024)          # workgroup units for small matrices
     if plan_split is not None:
-        assert op.info.plan_split_nz == min(plan_split, op.info.plan_unit_nz)
+        # a wavefront never takes more than one unit; a workgroup takes whole rows up to the threshold
+        assert op.info.plan_split_nz == (plan_split if op.info.plan_team else min(plan_split, op.info.plan_unit_nz))
     if plan_unit is not None:
         assert op.info.plan_unit_nz == plan_unit
     assert op.info.plan_groups == (plan_groups or 0)
@@ -182,9 +188,10 @@ def test_call_order_and_arguments(gpu):
 def check_plan(op, n_cols):
     """The launch plan covers every non-zero exactly once; units of whole rows stay
     inside one block4 entry and hold at most plan_unit non-zeros (or one row); pieces of
-    split rows hold at most plan_unit non-zeros of one column group and are queued on the
-    die that owns that group."""
+    split rows hold at most plan_unit non-zeros (the split threshold, if that is larger)
+    of one column group and are queued on the die that owns that group."""
     unit, split = op.info.plan_unit_nz, op.info.plan_split_nz
+    piece = max(unit, split)
     plan = op.plan().astype(np.int64)
     b4 = op.block4().astype(np.int64)
     sip, six, _ = op.sorted_csr()
@@ -196,7 +203,7 @@ def check_plan(op, n_cols):
     covered = np.zeros(six.size, dtype=np.int32)
     for x, y, z, w in long_:
         covered[z:z + w] += 1
-        assert 0 < w <= unit and sip[y] <= z and z + w <= sip[y + 1] and deg[y] > split
+        assert 0 < w <= piece and sip[y] <= z and z + w <= sip[y + 1] and deg[y] > split
     entry_of_row = {}
     for d, r, loc, info in b4[b4[:, 0] <= 384]:
         for q in range(info & 0xFFFF):
@@ -233,10 +240,12 @@ def check_plan(op, n_cols):
         assert max(per_queue) - min(per_queue) <= 1               # queues are level
 
 
+@pytest.mark.parametrize("team", [1, 2])
 @pytest.mark.parametrize("seed,n_long", [(0, 0), (1, 3), (2, 9)])
-def test_launch_plan(gpu, seed, n_long):
+def test_launch_plan(gpu, seed, n_long, team):
     g = helpers.graph_from_degrees(helpers.degree_mix(seed=seed, n_long=n_long), seed=seed)
-    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_team=team)
+    assert (op.info.plan_unit_nz, op.info.plan_split_nz) == ((48, 384) if team == 2 else (48, 48))
     check_plan(op, g.n_cols)
     op.close()
 
@@ -265,13 +274,14 @@ def test_plan_column_groups(gpu, groups):
     assert e.value.status == gpu._lib.ERR_ARG
 
 
+@pytest.mark.parametrize("team", [1, 2])
 @pytest.mark.parametrize("unit", [16, 50, 96, 200, 384])
-def test_plan_unit_sizes(gpu, unit):
+def test_plan_unit_sizes(gpu, unit, team):
     """Smaller units change the plan and which rows are stored grouped, never the
-    block4 metadata or the product."""
+    block4 metadata or the product; with a wavefront or a workgroup per unit."""
     from oracle import spmm_oracle as so
     g = helpers.graph_from_degrees(helpers.degree_mix(seed=6, n_long=5), seed=6)
-    op = check_preprocess(gpu, g, plan_unit=unit)
+    op = check_preprocess(gpu, g, plan_unit=unit, plan_team=team)
     check_plan(op, g.n_cols)
     for N in (64, 10):
         X = np.random.default_rng(unit + N).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
@@ -281,6 +291,9 @@ def test_plan_unit_sizes(gpu, unit):
     op.close()
     with pytest.raises(gpu.AccelError) as e:
         gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_unit=1000)
+    assert e.value.status == gpu._lib.ERR_ARG
+    with pytest.raises(gpu.AccelError) as e:
+        gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_team=3)
     assert e.value.status == gpu._lib.ERR_ARG
 
 
@@ -298,11 +311,12 @@ def test_plan_groups_follow_row_length(gpu):
     op.close()
 
 
+@pytest.mark.parametrize("team", [1, 2])
 @pytest.mark.parametrize("unit,split", [(384, 100), (384, 200), (128, 40), (96, 384)])
-def test_plan_split_threshold(gpu, unit, split):
+def test_plan_split_threshold(gpu, unit, split, team):
     from oracle import spmm_oracle as so
     g = helpers.graph_from_degrees(helpers.degree_mix(seed=9, n_long=6), seed=9)
-    op = check_preprocess(gpu, g, plan_unit=unit, plan_split=split)
+    op = check_preprocess(gpu, g, plan_unit=unit, plan_split=split, plan_team=team)
     check_plan(op, g.n_cols)
     X = np.random.default_rng(split).uniform(-1, 1, (g.n_cols, 40)).astype(np.float32)
     assert so.check(op.matmul(X), g.indptr, g.indices, g.values, X) <= so.TOL

@@ -16,10 +16,15 @@ TOL = 1e-5
 ALL_N = [1, 2, 3, 4, 5, 6, 8, 12, 16, 17, 30, 32, 48, 60, 64, 100, 128, 130, 200, 256, 260, 300, 512, 515]
 
 
-@pytest.fixture(scope="module")
-def mixed(gpu):
+@pytest.fixture(scope="module", params=["workgroup units", "wavefront units"])
+def mixed(gpu, request):
+    """A small matrix with every degree regime, once with a workgroup per unit (what the
+    library chooses for a matrix of this size) and once with a wavefront per unit (what
+    it chooses for large ones)."""
     g = helpers.graph_from_degrees(helpers.degree_mix(seed=7, n_long=8, zeros=11), seed=7)
-    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    team = 2 if request.param == "workgroup units" else 1
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_team=team)
+    assert op.info.plan_team == (team == 2)
     yield g, op
     op.close()
 
@@ -293,7 +298,8 @@ def test_operands_beyond_4_gib(gpu):
 def test_random_shapes(gpu):
     """Sixty seeded random matrices: random row counts, degree mixes (empty rows,
     every slice-table regime, rows of several thousand non-zeros) and column
-    counts 1..320, rectangular as well as square."""
+    counts 1..320, rectangular as well as square; alternately with a workgroup and
+    with a wavefront per unit."""
     rng = np.random.default_rng(2024)
     pool = np.array([0, 0, 1, 1, 2, 3, 7, 12, 31, 32, 33, 64, 65, 96, 97, 128, 129, 191, 192, 200, 383, 384,
                      385, 500, 768, 769, 1153, 3000])
@@ -306,7 +312,7 @@ def test_random_shapes(gpu):
         N = int(rng.integers(1, 321))
         g = gpu.synthetic.random_csr(n_rows, n_cols, deg, seed=case)
         X = rng.uniform(-1, 1, (n_cols, N)).astype(np.float32)
-        op = gpu.AccelSpMM(g.indptr, g.indices, g.values, n_cols).preprocess()
+        op = gpu.AccelSpMM(g.indptr, g.indices, g.values, n_cols).preprocess(plan_team=1 + case % 2)
         Y = op.matmul(X)
         assert np.isfinite(Y).all(), (case, n_rows, N)
         err = so.check(Y, g.indptr, g.indices, g.values, X)
