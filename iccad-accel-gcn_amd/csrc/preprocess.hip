@@ -301,22 +301,56 @@ __global__ __launch_bounds__(kThreads) void iota_kernel(uint32_t *out, int64_t n
 // Permuted CSR: non-zero p of the sorted matrix comes from the caller's row
 // perm[r], where r is the sorted row that contains p.
 // ---------------------------------------------------------------------------
+constexpr int kPermuteNz = 4;                        // non-zeros per thread
+constexpr int kPermuteTile = kThreads * kPermuteNz;  // non-zeros per workgroup
+
+// A workgroup copies kPermuteTile consecutive non-zeros of the sorted matrix.  They belong
+// to at most kPermuteTile + 1 consecutive sorted rows (rows without non-zeros all precede
+// the first non-zero), whose boundaries and source offsets are put in LDS once; each
+// thread then finds the row of its non-zeros by a search in LDS.
 __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
     const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
     const float *__restrict__ val, const int32_t *__restrict__ perm,
     const int32_t *__restrict__ s_indptr, int64_t rows, int64_t n_take, int32_t *__restrict__ s_idx,
     float *__restrict__ s_val)
 {
-    const int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    if (p >= n_take) return;
-    int64_t lo = 0, hi = rows - 1;  // first row whose end is beyond p
-    while (lo < hi) {
-        const int64_t mid = (lo + hi) >> 1;
-        if ((int64_t)s_indptr[mid + 1] > p) hi = mid; else lo = mid + 1;
+    __shared__ int row_end[kPermuteTile + 1];        // s_indptr[first + j + 1]
+    __shared__ int64_t shift[kPermuteTile + 1];      // source position minus sorted position, per row
+    __shared__ int64_t first_row_s;
+    const int64_t p0 = (int64_t)blockIdx.x * kPermuteTile;
+    const int64_t p1 = min(p0 + kPermuteTile, n_take);   // this workgroup copies [p0, p1)
+    if (threadIdx.x == 0) {
+        int64_t lo = 0, hi = rows - 1;               // first row whose end is beyond p0
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if ((int64_t)s_indptr[mid + 1] > p0) hi = mid; else lo = mid + 1;
+        }
+        first_row_s = lo;
     }
-    const int64_t src = (int64_t)indptr[perm ? perm[lo] : lo] + (p - s_indptr[lo]);
-    s_idx[p] = idx[src];
-    s_val[p] = val[src];
+    __syncthreads();
+    const int64_t first_row = first_row_s;
+    // rows first_row .. first_row + n_here - 1 cover [p0, p1): every one of them but the last ends
+    // inside the range, and each holds at least one non-zero, so n_here <= p1 - p0 + 1
+    const int n_max = (int)min((int64_t)kPermuteTile + 1, rows - first_row);
+    for (int j = threadIdx.x; j < n_max; j += kThreads) {
+        const int64_t r = first_row + j;
+        row_end[j] = s_indptr[r + 1];
+        shift[j] = (int64_t)indptr[perm ? perm[r] : r] - (int64_t)s_indptr[r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < kPermuteNz; q++) {
+        const int64_t p = p0 + (int64_t)q * kThreads + threadIdx.x;
+        if (p >= p1) break;
+        int lo = 0, hi = n_max - 1;                  // first j with row_end[j] > p
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if ((int64_t)row_end[mid] > p) hi = mid; else lo = mid + 1;
+        }
+        const int64_t src = p + shift[lo];
+        s_idx[p] = idx[src];
+        s_val[p] = val[src];
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -572,21 +606,65 @@ __global__ __launch_bounds__(kThreads) void emit_short_units_kernel(
     }
 }
 
-struct DevBuf {  // frees on scope exit
+// Temporaries of one preprocessing call come out of a few large device allocations
+// instead of one hipMalloc / hipFree each (a pair costs about 0.2 ms, and there are
+// some twenty temporaries).  Chunks are freed when the arena goes out of scope.
+struct Arena {
+    static constexpr int kMaxChunks = 32;
+    char *chunk[kMaxChunks] = {};
+    size_t cap = 0, used = 0;      // of the newest chunk
+    int n_chunks = 0;
+    size_t next_chunk = 0;         // size hint for the next chunk
+    ~Arena()
+    {
+        for (int i = 0; i < n_chunks; i++) (void)hipFree(chunk[i]);
+    }
+    void *take(size_t bytes)
+    {
+        bytes = (std::max<size_t>(bytes, 4) + 255) & ~(size_t)255;
+        if (n_chunks == 0 || used + bytes > cap) {
+            if (n_chunks == kMaxChunks) return nullptr;
+            const size_t want = std::max(bytes, next_chunk);
+            void *p = nullptr;
+            if (hipMalloc(&p, want) != hipSuccess) {
+                (void)hipGetLastError();
+                return nullptr;
+            }
+            chunk[n_chunks++] = static_cast<char *>(p);
+            cap = want;
+            used = 0;
+            next_chunk = std::max<size_t>(next_chunk / 4, (size_t)1 << 20);   // later chunks: leftovers only
+        }
+        void *p = chunk[n_chunks - 1] + used;
+        used += bytes;
+        return p;
+    }
+};
+
+struct DevBuf {  // frees on scope exit; with an arena, the arena owns the memory
     void *p = nullptr;
-    ~DevBuf() { if (p) (void)hipFree(p); }
+    Arena *arena = nullptr;
+    DevBuf() = default;
+    explicit DevBuf(Arena *a) : arena(a) {}
+    DevBuf(const DevBuf &) = delete;
+    DevBuf &operator=(const DevBuf &) = delete;
+    ~DevBuf() { if (p && !arena) (void)hipFree(p); }
     int alloc(size_t bytes)
     {
-        if (hipMalloc(&p, bytes ? bytes : 4) != hipSuccess) {
+        if (arena) {
+            p = arena->take(bytes);
+        } else if (hipMalloc(&p, bytes ? bytes : 4) != hipSuccess) {
             p = nullptr;
             (void)hipGetLastError();
+        }
+        if (!p) {
             set_error("device allocation of %zu bytes failed", bytes);
             return ACCEL_ERR_ALLOC;
         }
         return ACCEL_OK;
     }
     template <class T> T *as() { return static_cast<T *>(p); }
-    void *release() { void *q = p; p = nullptr; return q; }
+    void *release() { void *q = p; p = nullptr; return q; }   // only for buffers without an arena
 };
 
 inline unsigned grid_for(int64_t n) { return (unsigned)((n + kThreads - 1) / kThreads); }
@@ -595,11 +673,11 @@ inline unsigned grid_for(int64_t n) { return (unsigned)((n + kThreads - 1) / kTh
 
 // Builds block4 from degrees given in partition order.  The output is a freshly
 // allocated device array (caller frees); *n_blocks is returned on the host.
-static int partition_device(const uint32_t *deg, const int32_t *s_indptr, int64_t rows,
+static int partition_device(Arena *tmp, const uint32_t *deg, const int32_t *s_indptr, int64_t rows,
                             int32_t **block4_out, int64_t *n_blocks, hipStream_t s,
                             int64_t probe_row = -1, int64_t *blocks_before_probe = nullptr)
 {
-    DevBuf head, cnt, sums, rb, b4;
+    DevBuf head(tmp), cnt(tmp), sums(tmp), rb(tmp), b4;
     int rc;
     if ((rc = head.alloc(sizeof(int) * (size_t)rows))) return rc;
     if ((rc = cnt.alloc(sizeof(int) * (size_t)rows))) return rc;
@@ -636,7 +714,9 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
                           int32_t **block4_dev, int64_t *n_blocks)
 {
     hipStream_t s = nullptr;
-    DevBuf deg, st;
+    Arena tmp;
+    tmp.next_chunk = (size_t)rows * 24 + (1 << 16);
+    DevBuf deg(&tmp), st(&tmp);
     int rc;
     if ((rc = deg.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
     if ((rc = st.alloc(sizeof(Stats)))) return rc;
@@ -650,7 +730,7 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
         set_error("indptr must start at 0, be non-decreasing and end at nnz");
         return ACCEL_ERR_CSR;
     }
-    return partition_device(deg.as<uint32_t>(), indptr_dev, rows, block4_dev, n_blocks, s);
+    return partition_device(&tmp, deg.as<uint32_t>(), indptr_dev, rows, block4_dev, n_blocks, s);
 }
 
 // The launch plan.  One work unit per wavefront, kWavesPerGroup units per
@@ -670,7 +750,7 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
 // highest degree first, until all queues are equally long.  While a die works
 // through one group its L2 only has to hold that group's share of X.  The host
 // sees 121 bin totals and one unit count, to size the queues.
-static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_indptr,
+static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const int32_t *s_indptr,
                            int64_t first_long, int64_t n_short, hipStream_t s)
 {
     // "long" here = rows cut into pieces (more than plan_split non-zeros); n_short = block4
@@ -678,7 +758,7 @@ static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_
     const int64_t n_long = h->n_split_rows;
     // pieces of split rows hold up to piece_nz non-zeros, units of several whole rows up to unit_nz
     const int unit_nz = h->plan_unit, piece_nz = std::max(h->plan_unit, h->plan_split), forced = h->plan_groups;
-    DevBuf row_units, grp_units, sums, totals, dslot, scnt;
+    DevBuf row_units(tmp), grp_units(tmp), sums(tmp), totals(tmp), dslot, scnt(tmp);
     int rc;
     int tot[kPlanBins + 1] = {0};
     if ((rc = dslot.alloc(sizeof(int) * (size_t)(n_long + 1)))) return rc;
@@ -708,7 +788,7 @@ static int build_work_list(accel_handle *h, const int *gcount, const int32_t *s_
     int n_short_units32 = 0;
     if ((rc = scnt.alloc(sizeof(int) * (size_t)(n_short + 1)))) return rc;
     if (n_short > 0) {
-        DevBuf ssums;
+        DevBuf ssums(tmp);
         if ((rc = ssums.alloc(sizeof(int) * (size_t)(n_short / kTile + 4)))) return rc;
         short_unit_count_kernel<<<dim3(grid_for(n_short)), dim3(kThreads), 0, s>>>(
             reinterpret_cast<const int4 *>(h->block4), (int)n_short, unit_nz, scnt.as<int>());
@@ -862,7 +942,11 @@ int preprocess_device(accel_handle *h)
         return ACCEL_OK;
     }
 
-    DevBuf deg, st;
+    // temporaries: about 40 bytes per row when the rows have to be sorted, 24 otherwise,
+    // plus what the split rows need; further chunks are added on demand
+    Arena tmp;
+    tmp.next_chunk = (size_t)rows * 44 + (size_t)(rows / kTile + 1) * 1100 + (1 << 20);
+    DevBuf deg(&tmp), st(&tmp);
     if ((rc = deg.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
     if ((rc = st.alloc(sizeof(Stats)))) return rc;
     ACCEL_HIP(hipMemsetAsync(st.p, 0, sizeof(Stats), s));
@@ -894,7 +978,7 @@ int preprocess_device(accel_handle *h)
     h->identity_perm = !hs.unsorted;
 
     // ---- degree sort ------------------------------------------------------
-    DevBuf keys_b, vals_a, vals_b, hist, sums;
+    DevBuf keys_b(&tmp), vals_a(&tmp), vals_b(&tmp), hist(&tmp), sums(&tmp);
     uint32_t *sdeg = deg.as<uint32_t>();
     uint32_t *perm = nullptr;
     if (!h->identity_perm) {
@@ -926,7 +1010,7 @@ int preprocess_device(accel_handle *h)
     }
 
     // ---- sorted indptr ------------------------------------------------------
-    DevBuf sip, ssums;
+    DevBuf sip, ssums(&tmp);
     if ((rc = sip.alloc(sizeof(int32_t) * (size_t)(rows + 1)))) return rc;
     if ((rc = ssums.alloc(sizeof(int) * (size_t)(rows / kTile + 4)))) return rc;
     if ((rc = device_scan<SumOp, false>(reinterpret_cast<const int *>(sdeg), rows, sip.as<int>(),
@@ -945,7 +1029,7 @@ int preprocess_device(accel_handle *h)
     ACCEL_HIP(hipStreamSynchronize(s));
     const int64_t nnz_short = nnz_short32;
     const bool own_copy = !h->identity_perm || n_long > 0;
-    DevBuf sidx, sval, permbuf, gcount;
+    DevBuf sidx, sval, permbuf, gcount(&tmp);
     if (own_copy) {
         if ((rc = sidx.alloc(sizeof(int32_t) * (size_t)nnz))) return rc;
         if ((rc = sval.alloc(sizeof(float) * (size_t)nnz))) return rc;
@@ -959,7 +1043,7 @@ int preprocess_device(accel_handle *h)
             }
         } else {
             if (nnz_short > 0)
-                permute_csr_kernel<<<dim3(grid_for(nnz_short)), dim3(kThreads), 0, s>>>(
+                permute_csr_kernel<<<dim3((unsigned)((nnz_short + kPermuteTile - 1) / kPermuteTile)), dim3(kThreads), 0, s>>>(
                     h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), rows, nnz_short,
                     sidx.as<int32_t>(), sval.as<float>());
             if ((rc = permbuf.alloc(sizeof(int32_t) * (size_t)rows))) return rc;
@@ -979,7 +1063,7 @@ int preprocess_device(accel_handle *h)
     int32_t *b4 = nullptr;
     int64_t nb = 0;
     int64_t n_short_entries = 0;   // block4 entries of the rows that are not cut into pieces
-    if ((rc = partition_device(sdeg, sip.as<int32_t>(), rows, &b4, &nb, s, first_long, &n_short_entries)))
+    if ((rc = partition_device(&tmp, sdeg, sip.as<int32_t>(), rows, &b4, &nb, s, first_long, &n_short_entries)))
         return rc;
     ACCEL_HIP(hipStreamSynchronize(s));
     h->block4 = b4;
@@ -990,7 +1074,7 @@ int preprocess_device(accel_handle *h)
     }
 
     // ---- work list ------------------------------------------------------------
-    if ((rc = build_work_list(h, gcount.as<int>(), sip.as<int32_t>(), first_long, n_short_entries, s)))
+    if ((rc = build_work_list(&tmp, h, gcount.as<int>(), sip.as<int32_t>(), first_long, n_short_entries, s)))
         return rc;
 
     h->s_indptr = static_cast<int32_t *>(sip.release());
