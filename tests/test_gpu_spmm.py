@@ -214,6 +214,52 @@ def test_medium_power_law_graph(gpu):
     op.close()
 
 
+@pytest.mark.parametrize("name,N,rows,min_nnz", [("cfg4", 64, 2_450_000, 120_000_000),
+                                                  ("cfg3", 64, 233_000, 110_000_000),
+                                                  ("cfg5", 256, 1_000_000, 25_000_000)])
+def test_large_workloads_at_full_size(gpu, name, N, rows, min_nnz):
+    """The three large benchmark workloads as benchmarked (cfg4 is the headline: 2.45 M rows,
+    ~125 M non-zeros, N = 64), checked through properties that cost O(nnz) on the host:
+    X = 1 gives the row sums of A; the column sums of Y equal (1^T A) X;
+    A (X1 + X2) = A X1 + A X2; the first rows against fp64."""
+    g = getattr(gpu.synthetic, name)()
+    assert g.n_rows == rows and g.nnz > min_nnz
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    assert op.info.plan_team == 0 and op.info.plan_unit_nz == 384
+    v64 = g.values.astype(np.float64)
+    filled = np.flatnonzero(np.diff(g.indptr) > 0)       # reduceat wants strictly increasing starts
+    row_sum, row_abs = np.zeros(g.n_rows), np.zeros(g.n_rows)
+    row_sum[filled] = np.add.reduceat(v64, g.indptr[filled].astype(np.int64))
+    row_abs[filled] = np.add.reduceat(np.abs(v64), g.indptr[filled].astype(np.int64))
+    tiny = 1e-300
+    ones = gpu.DeviceBuffer.from_numpy(np.ones((g.n_cols, N), np.float32))
+    dY = gpu.DeviceBuffer(g.n_rows * N * 4)
+    op.run(ones, dY, N)
+    Y1 = dY.to_numpy(np.float32, (g.n_rows, N))
+    assert np.max(np.abs(Y1 - row_sum[:, None]) / np.maximum(row_abs[:, None], tiny)) <= TOL
+    ones.close()
+    dY.close()
+    del Y1
+    X1 = gpu.synthetic.dense_operand(name, g.n_cols, N)
+    X2 = np.random.default_rng(5).uniform(-1, 1, X1.shape).astype(np.float32)
+    col_w = np.bincount(g.indices, weights=v64, minlength=g.n_cols)
+    col_a = np.bincount(g.indices, weights=np.abs(v64), minlength=g.n_cols)
+    Ya = op.matmul(X1)
+    check_sum = Ya.sum(axis=0, dtype=np.float64)
+    bound = col_a @ np.abs(X1).astype(np.float64)
+    assert np.max(np.abs(check_sum - col_w @ X1.astype(np.float64)) / np.maximum(bound, tiny)) <= TOL
+    head = int(np.searchsorted(g.indptr, 2_000_000))     # rows holding the first ~2 M non-zeros
+    nz = int(g.indptr[head])
+    R, S = so.spmm_fp64(g.indptr[: head + 1], g.indices[:nz], g.values[:nz], X1)
+    assert so.scaled_error(Ya[:head], R, S) <= TOL
+    Yb = op.matmul(X2)
+    Yc = op.matmul(X1 + X2)
+    # |A| (|X1| + |X2|) <= |A| 1 (max|X1| + max|X2|)
+    Sabs = row_abs[:, None] * float(np.abs(X1).max() + np.abs(X2).max())
+    assert np.max(np.abs(Yc - (Ya + Yb)) / np.maximum(Sabs, tiny)) <= 4 * TOL
+    op.close()
+
+
 @pytest.mark.parametrize("N", [16, 64, 100, 3])
 def test_fused_bias_and_relu(gpu, mixed, N):
     """Y = relu(A X + b) in the store; rows of degree 0 become relu(b)."""
