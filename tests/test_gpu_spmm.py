@@ -366,6 +366,21 @@ def test_random_shapes(gpu):
         op.close()
 
 
+def test_very_wide_operand(gpu):
+    """N beyond 8192 columns: many column passes per unit, and the zero-fill of empty rows
+    changes from several rows per workgroup to one."""
+    deg = np.array([0, 3, 0, 40, 500, 1, 0, 200, 12, 0, 385], dtype=np.int64)
+    g = helpers.graph_from_degrees(deg, n_cols=600, seed=12)
+    for team in (1, 2):
+        op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_team=team)
+        for N in (8188, 8192, 8200, 9001):
+            X = np.random.default_rng(N).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+            Y = op.matmul(X)
+            assert np.all(Y[deg == 0] == 0.0)
+            assert so.check(Y, g.indptr, g.indices, g.values, X) <= TOL, (team, N)
+        op.close()
+
+
 def test_column_panels(gpu):
     """Wide operands on a matrix large enough to be computed in 64-column panels
     (N = 128, 256) next to widths that are not (N = 100, 192 is, 130 is not)."""

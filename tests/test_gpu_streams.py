@@ -58,6 +58,38 @@ def test_two_streams_two_handles(gpu, hip):
     ok(hip.hipStreamDestroy(s2))
 
 
+def test_two_host_threads_two_handles(gpu):
+    """Distinct handles are independent: two host threads create, preprocess, run and
+    check their own operator at the same time; errors are reported per thread."""
+    import threading
+    results, errors = {}, {}
+
+    def worker(tag, seed, N):
+        try:
+            for rep in range(3):
+                g, X, op = make_case(gpu, seed + rep, N)
+                Y = op.matmul(X)
+                results[(tag, rep)] = so.check(Y, g.indptr, g.indices, g.values, X)
+                op.close()
+            # an error on this thread must not show up as the other thread's message
+            with pytest.raises(gpu.AccelError) as e:
+                gpu.AccelSpMM(np.array([0, 2, 1], np.int32), np.zeros(1, np.int32), np.zeros(1, np.float32), 4)\
+                    .preprocess()
+            errors[tag] = str(e.value)
+        except BaseException as exc:                      # surfaced by the assertions below
+            errors[tag] = f"worker failed: {exc!r}"
+
+    threads = [threading.Thread(target=worker, args=("a", 40, 64)),
+               threading.Thread(target=worker, args=("b", 50, 24))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+        assert not t.is_alive()
+    assert len(results) == 6 and all(v <= so.TOL for v in results.values()), (results, errors)
+    assert all("indptr" in errors[t] for t in ("a", "b")), errors
+
+
 def test_graph_capture_and_replay(gpu, hip):
     g, X, op = make_case(gpu, 33, 64)
     N = 64
