@@ -66,12 +66,14 @@ def cpu_baseline(g, X, N, budget_s=15.0):
                       f"({nz} of {g.nnz} non-zeros), N={N}, 1 thread"}, n_rows, Y
 
 
-def fixture_graph(pkg, name, seed=0):
+def fixture_graph(pkg, name, seed=0, sigma=0):
     """A graph with exactly the degree sequence of one of the reference's
     benchmark graphs (recovered from its golden .block4 metadata: degree, first
     row and row count of every block; rows no block covers have degree 0), rows
-    in shuffled order, columns uniform random (distinct inside a row), values
-    GCN-normalised.  The real edge lists are not available offline."""
+    in shuffled order, values GCN-normalised.  The real edge lists are not
+    available offline, so the columns are synthetic: uniform random (sigma = 0),
+    or, to model a vertex order with locality, row id + N(0, sigma) (duplicates
+    inside a row merge, so such a graph has slightly fewer non-zeros)."""
     sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "golden"))
     import block4_codec
     b = block4_codec.load(name).astype(np.int64)
@@ -86,7 +88,10 @@ def fixture_graph(pkg, name, seed=0):
     rng = np.random.default_rng(seed)
     deg = rng.permutation(deg)
     src = np.repeat(np.arange(n, dtype=np.int64), deg)
-    dst = rng.integers(0, n, size=src.size, dtype=np.int64)
+    if sigma > 0:
+        dst = np.clip(src + np.rint(rng.standard_normal(src.size) * sigma).astype(np.int64), 0, n - 1)
+    else:
+        dst = rng.integers(0, n, size=src.size, dtype=np.int64)
     syn = pkg.synthetic
     indptr, indices = syn._csr_from_edges(src, dst, n, n)
     g = syn.Graph(name, indptr, indices, syn._gcn_values(indptr, indices), n, n)
@@ -154,7 +159,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--workload", default="cfg4",
                     help="cfg1..cfg5, or fixture:<name> for the degree sequence of one of the "
-                         "reference's graphs (e.g. fixture:OVCAR-8H, fixture:ppa)")
+                         "reference's graphs (e.g. fixture:OVCAR-8H, fixture:ppa) with uniform random "
+                         "columns, or local:<name>:<sigma> for the same with columns within about "
+                         "sigma of the row id")
     ap.add_argument("--N", type=int, default=0, help="columns of X (default: the workload's first)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the scipy baseline and the check")
     ap.add_argument("--compare-rocsparse", action="store_true",
@@ -191,6 +198,9 @@ def main():
     t0 = time.time()
     if a.workload.startswith("fixture:"):
         g = fixture_graph(pkg, a.workload.split(":", 1)[1])
+    elif a.workload.startswith("local:"):               # local:<name>:<sigma>
+        _, name, sigma = a.workload.split(":")
+        g = fixture_graph(pkg, name, sigma=int(sigma))
     elif a.workload in syn.WORKLOADS:
         g = syn.WORKLOADS[a.workload]()
     else:

@@ -297,6 +297,109 @@ __global__ __launch_bounds__(kThreads) void iota_kernel(uint32_t *out, int64_t n
     if (i < n) out[i] = (uint32_t)i;
 }
 
+// Temporaries of one preprocessing call come out of a few large device allocations
+// instead of one hipMalloc / hipFree each (a pair costs about 0.2 ms, and there are
+// some twenty temporaries).  Chunks are freed when the arena goes out of scope.
+struct Arena {
+    static constexpr int kMaxChunks = 32;
+    char *chunk[kMaxChunks] = {};
+    size_t cap = 0, used = 0;      // of the newest chunk
+    int n_chunks = 0;
+    size_t next_chunk = 0;         // size hint for the next chunk
+    ~Arena()
+    {
+        for (int i = 0; i < n_chunks; i++) (void)hipFree(chunk[i]);
+    }
+    void *take(size_t bytes)
+    {
+        bytes = (std::max<size_t>(bytes, 4) + 255) & ~(size_t)255;
+        if (n_chunks == 0 || used + bytes > cap) {
+            if (n_chunks == kMaxChunks) return nullptr;
+            const size_t want = std::max(bytes, next_chunk);
+            void *p = nullptr;
+            if (hipMalloc(&p, want) != hipSuccess) {
+                (void)hipGetLastError();
+                return nullptr;
+            }
+            chunk[n_chunks++] = static_cast<char *>(p);
+            cap = want;
+            used = 0;
+            next_chunk = std::max<size_t>(next_chunk / 4, (size_t)1 << 20);   // later chunks: leftovers only
+        }
+        void *p = chunk[n_chunks - 1] + used;
+        used += bytes;
+        return p;
+    }
+};
+
+struct DevBuf {  // frees on scope exit; with an arena, the arena owns the memory
+    void *p = nullptr;
+    Arena *arena = nullptr;
+    DevBuf() = default;
+    explicit DevBuf(Arena *a) : arena(a) {}
+    DevBuf(const DevBuf &) = delete;
+    DevBuf &operator=(const DevBuf &) = delete;
+    ~DevBuf() { if (p && !arena) (void)hipFree(p); }
+    int alloc(size_t bytes)
+    {
+        if (arena) {
+            p = arena->take(bytes);
+        } else if (hipMalloc(&p, bytes ? bytes : 4) != hipSuccess) {
+            p = nullptr;
+            (void)hipGetLastError();
+        }
+        if (!p) {
+            set_error("device allocation of %zu bytes failed", bytes);
+            return ACCEL_ERR_ALLOC;
+        }
+        return ACCEL_OK;
+    }
+    template <class T> T *as() { return static_cast<T *>(p); }
+    void *release() { void *q = p; p = nullptr; return q; }   // only for buffers without an arena
+};
+
+inline unsigned grid_for(int64_t n) { return (unsigned)((n + kThreads - 1) / kThreads); }
+
+// Sorts n (key, position) pairs by key, stably, in as many 8-bit passes as max_key needs.
+// keys is used as one of the two key buffers; *sorted_keys / *sorted_vals point at the
+// results (vals = original positions).  With max_key == 0 nothing moves.
+int radix_sort_pairs(Arena *tmp, uint32_t *keys, int64_t n, uint32_t max_key, hipStream_t s,
+                     uint32_t **sorted_keys, uint32_t **sorted_vals)
+{
+    DevBuf keys_b(tmp), vals_a(tmp), vals_b(tmp), hist(tmp), sums(tmp);
+    const int64_t tiles = (n + kTile - 1) / kTile;
+    int rc;
+    if ((rc = keys_b.alloc(sizeof(uint32_t) * (size_t)n))) return rc;
+    if ((rc = vals_a.alloc(sizeof(uint32_t) * (size_t)n))) return rc;
+    if ((rc = vals_b.alloc(sizeof(uint32_t) * (size_t)n))) return rc;
+    if ((rc = hist.alloc(sizeof(int) * (size_t)(256 * tiles)))) return rc;
+    if ((rc = sums.alloc(sizeof(int) * (size_t)(256 * tiles / kTile + 4)))) return rc;
+    int bits = 0;
+    while (bits < 32 && (max_key >> bits) != 0) bits++;
+    uint32_t *kin = keys, *kout = keys_b.as<uint32_t>();
+    uint32_t *vin = nullptr, *vout = vals_a.as<uint32_t>();
+    for (int shift = 0; shift < bits; shift += 8) {
+        radix_hist<<<dim3((unsigned)tiles), dim3(kThreads), 0, s>>>(kin, n, shift, hist.as<int>(), tiles);
+        if ((rc = device_scan<SumOp, false>(hist.as<int>(), 256 * tiles, hist.as<int>(), nullptr,
+                                            sums.as<int>(), s)))
+            return rc;
+        radix_scatter<<<dim3((unsigned)tiles), dim3(kThreads), 0, s>>>(kin, vin, kout, vout, n, shift,
+                                                                     hist.as<int>(), tiles);
+        std::swap(kin, kout);
+        vin = vout;
+        vout = (vout == vals_a.as<uint32_t>()) ? vals_b.as<uint32_t>() : vals_a.as<uint32_t>();
+    }
+    if (!vin) {                                        // no pass ran: positions in order
+        iota_kernel<<<dim3((unsigned)((n + kThreads - 1) / kThreads)), dim3(kThreads), 0, s>>>(
+            vals_a.as<uint32_t>(), n);
+        vin = vals_a.as<uint32_t>();
+    }
+    ACCEL_HIP(hipGetLastError());
+    *sorted_keys = kin;
+    *sorted_vals = vin;
+    return ACCEL_OK;
+}
+
 // ---------------------------------------------------------------------------
 // Permuted CSR: non-zero p of the sorted matrix comes from the caller's row
 // perm[r], where r is the sorted row that contains p.
@@ -481,7 +584,6 @@ __global__ __launch_bounds__(kThreads) void emit_block4_kernel(
 // ---------------------------------------------------------------------------
 struct PlanParams {
     int queue_long[kXcds];   // long-row units already in each queue
-    int quota[kXcds];        // units of whole rows each queue takes
 };
 struct BinOffsets {
     int off[kPlanBins];      // where the pieces of a (row class, column group) bin start in their queue
@@ -493,11 +595,28 @@ __device__ __forceinline__ int64_t plan_index(int queue, int pos)
     return ((int64_t)(pos / kWavesPerGroup) * kXcds + queue) * kWavesPerGroup + pos % kWavesPerGroup;
 }
 
-// grp_units is laid out [bin][split row, largest first] and must be zero on entry.
+// The split rows in the order of the caller's row ids: key[lr] = that id, and, after the
+// sort, rank[order[i]] = i.
+__global__ __launch_bounds__(kThreads) void long_row_key_kernel(const uint32_t *__restrict__ perm,
+                                                                int64_t first_long, int n_long,
+                                                                uint32_t *__restrict__ key)
+{
+    const int lr = blockIdx.x * kThreads + threadIdx.x;
+    if (lr < n_long) key[lr] = perm ? perm[first_long + lr] : (uint32_t)(first_long + lr);
+}
+
+__global__ __launch_bounds__(kThreads) void invert_order_kernel(const uint32_t *__restrict__ order, int n,
+                                                                int *__restrict__ rank)
+{
+    const int i = blockIdx.x * kThreads + threadIdx.x;
+    if (i < n) rank[order[i]] = i;
+}
+
+// grp_units is laid out [bin][split row, by rank] and must be zero on entry.
 __global__ __launch_bounds__(kThreads) void long_unit_count_kernel(
     const int *__restrict__ gcount, const int32_t *__restrict__ s_indptr, int64_t first_long,
-    int n_long, int forced_groups, int piece, int *__restrict__ row_units,
-    int *__restrict__ grp_units)
+    int n_long, int forced_groups, int piece, const int *__restrict__ rank,
+    int *__restrict__ row_units, int *__restrict__ grp_units)
 {
     const int lr = blockIdx.x * kThreads + threadIdx.x;
     if (lr >= n_long) return;
@@ -505,7 +624,7 @@ __global__ __launch_bounds__(kThreads) void long_unit_count_kernel(
     int tot = 0;
     for (int g = 0; g < ng; g++) {
         const int u = (gcount[(int64_t)lr * kMaxGroups + g] + piece - 1) / piece;
-        grp_units[(int64_t)plan_bin(ng, g) * n_long + (n_long - 1 - lr)] = u;   // largest rows first
+        grp_units[(int64_t)plan_bin(ng, g) * n_long + rank[lr]] = u;
         tot += u;
     }
     row_units[lr] = tot;
@@ -520,7 +639,7 @@ __global__ void plan_totals_kernel(const int *__restrict__ grp_pos, int n_long, 
 __global__ __launch_bounds__(kThreads) void emit_long_units_kernel(
     const int *__restrict__ gcount, const int32_t *__restrict__ s_indptr, int64_t first_long,
     const int *__restrict__ slot, const int *__restrict__ grp_pos, int n_long, int forced_groups,
-    int piece, BinOffsets bo, int4 *__restrict__ work)
+    int piece, const int *__restrict__ rank, BinOffsets bo, int4 *__restrict__ work)
 {
     const int t = blockIdx.x * kThreads + threadIdx.x;
     if (t >= n_long * kMaxGroups) return;
@@ -538,7 +657,7 @@ __global__ __launch_bounds__(kThreads) void emit_long_units_kernel(
     }
     const int loc = s_indptr[row] + c_before;
     const int bin = plan_bin(ng, g);
-    const int pos0 = bo.off[bin] + grp_pos[(int64_t)bin * n_long + (n_long - 1 - lr)] -
+    const int pos0 = bo.off[bin] + grp_pos[(int64_t)bin * n_long + rank[lr]] -
                      grp_pos[(int64_t)bin * n_long];
     const int sl = slot[lr] + u_before;
     for (int k = 0, off = 0; off < c; k++, off += piece)
@@ -549,125 +668,115 @@ __global__ __launch_bounds__(kThreads) void emit_long_units_kernel(
 // Rows a unit of whole rows may hold: as many as fit plan_unit non-zeros, at least one.
 __device__ __forceinline__ int rows_per_unit(int d, int unit_nz) { return max(1, unit_nz / d); }
 
-// Entries are visited from the last (highest degree) to the first; cnt[j] is the number
-// of units entry n_short - 1 - j is cut into.
+// cnt[j] = number of units block4 entry j (of the rows that are not split) is cut into.
 __global__ __launch_bounds__(kThreads) void short_unit_count_kernel(
     const int4 *__restrict__ block4, int n_short, int unit_nz, int *__restrict__ cnt)
 {
     const int j = blockIdx.x * kThreads + threadIdx.x;
     if (j >= n_short) return;
-    const int4 b = block4[n_short - 1 - j];
+    const int4 b = block4[j];
     const int n_rows = b.w & 0xFFFF, rpu = rows_per_unit(b.x, unit_nz);
     cnt[j] = (n_rows + rpu - 1) / rpu;
 }
 
-__device__ __forceinline__ void deal_position(int i, const PlanParams &pp, int &queue, int &pos)
+// What a unit costs, for levelling the queues: a gathered row of X per non-zero, a
+// written row of Y per row, a fixed part; scaled down (shift >= 2) so that the sum over
+// the matrix stays below 2^31.  (Counting units, or fixed parts of 64 or 200, measured the
+// same within noise.)
+__device__ __forceinline__ int unit_cost(int nz, int n_rows, int shift)
 {
-    // units are dealt in rounds; in round t every queue with quota > t takes one,
-    // in queue order.  dealt(t) = sum_q min(quota_q, t) units precede round t.
-    int lo = 0, hi = 0;
-#pragma unroll
-    for (int q = 0; q < kXcds; q++) hi = max(hi, pp.quota[q]);
-    while (lo < hi) {                                  // largest t with dealt(t) <= i
-        const int mid = (lo + hi + 1) >> 1;
-        int dealt = 0;
-#pragma unroll
-        for (int q = 0; q < kXcds; q++) dealt += min(pp.quota[q], mid);
-        if (dealt <= i) lo = mid; else hi = mid - 1;
-    }
-    int j = i;
-#pragma unroll
-    for (int q = 0; q < kXcds; q++) j -= min(pp.quota[q], lo);
-    queue = 0;
-#pragma unroll
-    for (int q = kXcds - 1; q >= 0; q--) {
-        // the j-th queue (ascending) that is still open in round lo
-        int open_before = 0;
-        for (int r = 0; r < q; r++) open_before += pp.quota[r] > lo;
-        if (pp.quota[q] > lo && open_before == j) queue = q;
-    }
-    pos = pp.queue_long[queue] + lo;
+    return ((nz + n_rows + 8) >> shift) + 1;
 }
 
-__global__ __launch_bounds__(kThreads) void emit_short_units_kernel(
+// Writes the units of whole rows in row order, and for each the caller's row id of its
+// first row: the key the units are queued by.
+__global__ __launch_bounds__(kThreads) void list_short_units_kernel(
     const int4 *__restrict__ block4, int n_short, int unit_nz, const int *__restrict__ first_unit,
-    PlanParams pp, int4 *__restrict__ work)
+    const uint32_t *__restrict__ perm, int4 *__restrict__ units, uint32_t *__restrict__ key)
 {
-    const int j = blockIdx.x * kThreads + threadIdx.x;   // dealing order: highest degree first
+    const int j = blockIdx.x * kThreads + threadIdx.x;
     if (j >= n_short) return;
-    const int4 b = block4[n_short - 1 - j];
+    const int4 b = block4[j];
     const int d = b.x, n_rows = b.w & 0xFFFF, w_nz = b.w >> 16, rpu = rows_per_unit(d, unit_nz);
     int i = first_unit[j];
     for (int r = 0; r < n_rows; r += rpu, i++) {
-        int queue, pos;
-        deal_position(i, pp, queue, pos);
-        work[plan_index(queue, pos)] =
-            make_int4(d, b.y + r, b.z + r * d, (w_nz << 16) + min(rpu, n_rows - r));
+        units[i] = make_int4(d, b.y + r, b.z + r * d, (w_nz << 16) + min(rpu, n_rows - r));
+        key[i] = perm ? perm[b.y + r] : (uint32_t)(b.y + r);
     }
 }
 
-// Temporaries of one preprocessing call come out of a few large device allocations
-// instead of one hipMalloc / hipFree each (a pair costs about 0.2 ms, and there are
-// some twenty temporaries).  Chunks are freed when the arena goes out of scope.
-struct Arena {
-    static constexpr int kMaxChunks = 32;
-    char *chunk[kMaxChunks] = {};
-    size_t cap = 0, used = 0;      // of the newest chunk
-    int n_chunks = 0;
-    size_t next_chunk = 0;         // size hint for the next chunk
-    ~Arena()
-    {
-        for (int i = 0; i < n_chunks; i++) (void)hipFree(chunk[i]);
-    }
-    void *take(size_t bytes)
-    {
-        bytes = (std::max<size_t>(bytes, 4) + 255) & ~(size_t)255;
-        if (n_chunks == 0 || used + bytes > cap) {
-            if (n_chunks == kMaxChunks) return nullptr;
-            const size_t want = std::max(bytes, next_chunk);
-            void *p = nullptr;
-            if (hipMalloc(&p, want) != hipSuccess) {
-                (void)hipGetLastError();
-                return nullptr;
-            }
-            chunk[n_chunks++] = static_cast<char *>(p);
-            cap = want;
-            used = 0;
-            next_chunk = std::max<size_t>(next_chunk / 4, (size_t)1 << 20);   // later chunks: leftovers only
+__global__ __launch_bounds__(kThreads) void short_unit_cost_kernel(
+    const int4 *__restrict__ units, const uint32_t *__restrict__ order, int n, int shift,
+    int light_nz, int *__restrict__ cost, int *__restrict__ heavy)
+{
+    const int sidx = blockIdx.x * kThreads + threadIdx.x;
+    if (sidx >= n) return;
+    const int4 u = units[order[sidx]];
+    const int n_rows = u.w & 0xFFFF;
+    cost[sidx] = unit_cost(u.x * n_rows, n_rows, shift);
+    heavy[sidx] = u.x * n_rows > light_nz;
+}
+
+// Non-zeros and pieces of the split rows per queue (column group g belongs to queue g % 8).
+__global__ __launch_bounds__(kThreads) void long_queue_load_kernel(
+    const int *__restrict__ gcount, int n_long, int piece, int shift, int *__restrict__ queue_cost)
+{
+    __shared__ int part[kXcds];
+    if (threadIdx.x < kXcds) part[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t t = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (t < (int64_t)n_long * kMaxGroups) {
+        const int c = gcount[t];
+        if (c > 0) {
+            const int pieces = (c + piece - 1) / piece;
+            atomicAdd(&part[(int)(t % kMaxGroups) % kXcds], ((c + 9 * pieces) >> shift) + pieces);
         }
-        void *p = chunk[n_chunks - 1] + used;
-        used += bytes;
-        return p;
     }
+    __syncthreads();
+    if (threadIdx.x < kXcds && part[threadIdx.x]) atomicAdd(&queue_cost[threadIdx.x], part[threadIdx.x]);
+}
+
+struct QueueCuts {
+    int cut[kXcds + 1];      // queue q takes the units whose running cost lies in [cut[q], cut[q + 1])
 };
 
-struct DevBuf {  // frees on scope exit; with an arena, the arena owns the memory
-    void *p = nullptr;
-    Arena *arena = nullptr;
-    DevBuf() = default;
-    explicit DevBuf(Arena *a) : arena(a) {}
-    DevBuf(const DevBuf &) = delete;
-    DevBuf &operator=(const DevBuf &) = delete;
-    ~DevBuf() { if (p && !arena) (void)hipFree(p); }
-    int alloc(size_t bytes)
-    {
-        if (arena) {
-            p = arena->take(bytes);
-        } else if (hipMalloc(&p, bytes ? bytes : 4) != hipSuccess) {
-            p = nullptr;
-            (void)hipGetLastError();
-        }
-        if (!p) {
-            set_error("device allocation of %zu bytes failed", bytes);
-            return ACCEL_ERR_ALLOC;
-        }
-        return ACCEL_OK;
-    }
-    template <class T> T *as() { return static_cast<T *>(p); }
-    void *release() { void *q = p; p = nullptr; return q; }   // only for buffers without an arena
-};
+__device__ __forceinline__ int queue_of(int running_cost, const QueueCuts &qc)
+{
+    int q = 0;
+#pragma unroll
+    for (int i = 1; i < kXcds; i++) q += running_cost >= qc.cut[i];
+    return q;
+}
 
-inline unsigned grid_for(int64_t n) { return (unsigned)((n + kThreads - 1) / kThreads); }
+// first[q] = rank of the first unit of queue q (n for queues that get none); first must hold n on entry.
+__global__ __launch_bounds__(kThreads) void queue_first_kernel(const int *__restrict__ running, int n,
+                                                               QueueCuts qc, int *__restrict__ first)
+{
+    const int sidx = blockIdx.x * kThreads + threadIdx.x;
+    if (sidx >= n) return;
+    const int q = queue_of(running[sidx], qc);
+    const int q_prev = sidx == 0 ? -1 : queue_of(running[sidx - 1], qc);
+    for (int i = q_prev + 1; i <= q; i++) first[i] = sidx;
+}
+
+// Inside its queue a unit goes behind the pieces; the units with many non-zeros first, the
+// light ones last (both in the order of the caller's row ids), so that a queue does not end
+// on a long chain of gathers.  heavy_before[s] = heavy units among the first s, [n] = all.
+__global__ __launch_bounds__(kThreads) void place_short_units_kernel(
+    const int4 *__restrict__ units, const uint32_t *__restrict__ order, const int *__restrict__ running,
+    const int *__restrict__ heavy_before, int n, QueueCuts qc, const int *__restrict__ first,
+    PlanParams pp, int4 *__restrict__ work)
+{
+    const int sidx = blockIdx.x * kThreads + threadIdx.x;
+    if (sidx >= n) return;
+    const int q = queue_of(running[sidx], qc);
+    const int f = first[q], f_next = first[q + 1];
+    const int h0 = heavy_before[f], h_all = heavy_before[f_next] - h0;     // heavy units of this queue
+    const int h_me = heavy_before[sidx] - h0;                              // ... before this unit
+    const bool is_heavy = heavy_before[sidx + 1] != heavy_before[sidx];
+    const int pos = is_heavy ? h_me : h_all + (sidx - f) - h_me;
+    work[plan_index(q, pp.queue_long[q] + pos)] = units[order[sidx]];
+}
 
 }  // namespace
 
@@ -744,23 +853,34 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
 // Workgroups are dispatched to the eight dies round-robin (workgroup i runs on
 // die i % 8), so the list is laid out as eight interleaved queues.  Column group
 // g belongs to die g % 8.  A queue holds, in this order: the pieces of the rows
-// stored in 64 groups (the longest rows), one group after the other, largest
-// rows first; then the same for the rows with 32, 16 and 8 groups; then the
-// queue's share of the whole-row units, which are dealt to the queues in rounds,
-// highest degree first, until all queues are equally long.  While a die works
-// through one group its L2 only has to hold that group's share of X.  The host
-// sees 121 bin totals and one unit count, to size the queues.
+// stored in 64 groups (the longest rows), one group after the other, the rows of
+// a group in the order of the caller's row ids; then the same for the rows with
+// 32, 16 and 8 groups; then the
+// queue's share of the whole-row units.  While a die works through one group its
+// L2 only has to hold that group's share of X.
+// The whole-row units are put in the order of the caller's row ids (of each unit's
+// first row) and that sequence is cut into eight consecutive shares, one per queue,
+// sized so that all queues carry about the same load.  Graphs whose neighbouring
+// row ids have neighbouring columns (most graphs with a meaningful vertex order)
+// lose that locality to the degree sort; this gives it back: at any time a die
+// works on a narrow band of the caller's rows.
+// The host sees 121 bin totals, eight queue loads, one unit count, one total cost
+// and nine share boundaries, to size the queues.
 static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const int32_t *s_indptr,
-                           int64_t first_long, int64_t n_short, hipStream_t s)
+                           int64_t first_long, int64_t n_short, const uint32_t *perm, hipStream_t s)
 {
     // "long" here = rows cut into pieces (more than plan_split non-zeros); n_short = block4
     // entries of all other rows (they precede the rest in block4)
     const int64_t n_long = h->n_split_rows;
     // pieces of split rows hold up to piece_nz non-zeros, units of several whole rows up to unit_nz
     const int unit_nz = h->plan_unit, piece_nz = std::max(h->plan_unit, h->plan_split), forced = h->plan_groups;
-    DevBuf row_units(tmp), grp_units(tmp), sums(tmp), totals(tmp), dslot, scnt(tmp);
+    DevBuf row_units(tmp), grp_units(tmp), sums(tmp), totals(tmp), dslot, scnt(tmp), qload(tmp), lkey(tmp),
+        lrank(tmp);
     int rc;
     int tot[kPlanBins + 1] = {0};
+    int long_cost[kXcds] = {0};
+    int cost_shift = 2;                                // total cost = about (nnz + 10 rows) >> shift + units < 2^31
+    while ((((int64_t)h->nnz + 10 * h->rows) >> cost_shift) + h->rows >= ((int64_t)1 << 30)) cost_shift++;
     if ((rc = dslot.alloc(sizeof(int) * (size_t)(n_long + 1)))) return rc;
     if (n_long > 0) {
         if ((rc = row_units.alloc(sizeof(int) * (size_t)n_long))) return rc;
@@ -768,10 +888,26 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         if ((rc = grp_units.alloc(sizeof(int) * (size_t)(n_bins + 1)))) return rc;
         if ((rc = sums.alloc(sizeof(int) * (size_t)(n_bins / kTile + 4)))) return rc;
         if ((rc = totals.alloc(sizeof(int) * (kPlanBins + 1)))) return rc;
+        if ((rc = qload.alloc(sizeof(int) * kXcds))) return rc;
         if ((rc = fill_u32(grp_units.p, 0u, (size_t)n_bins + 1, s))) return rc;
+        if ((rc = fill_u32(qload.p, 0u, kXcds, s))) return rc;
+        // inside a (row class, column group) bin the rows follow the caller's row ids, like the
+        // whole-row units further down
+        uint32_t *lkey_sorted = nullptr, *lorder = nullptr;
+        if ((rc = lkey.alloc(sizeof(uint32_t) * (size_t)n_long))) return rc;
+        if ((rc = lrank.alloc(sizeof(int) * (size_t)n_long))) return rc;
+        long_row_key_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(perm, first_long, (int)n_long,
+                                                                             lkey.as<uint32_t>());
+        if ((rc = radix_sort_pairs(tmp, lkey.as<uint32_t>(), n_long, (uint32_t)std::max<int64_t>(h->rows - 1, 0),
+                                   s, &lkey_sorted, &lorder)))
+            return rc;
+        invert_order_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(lorder, (int)n_long,
+                                                                             lrank.as<int>());
         long_unit_count_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(
-            gcount, s_indptr, first_long, (int)n_long, forced, piece_nz, row_units.as<int>(),
-            grp_units.as<int>());
+            gcount, s_indptr, first_long, (int)n_long, forced, piece_nz, lrank.as<int>(),
+            row_units.as<int>(), grp_units.as<int>());
+        long_queue_load_kernel<<<dim3(grid_for(n_long * kMaxGroups)), dim3(kThreads), 0, s>>>(
+            gcount, (int)n_long, piece_nz, cost_shift, qload.as<int>());
         if ((rc = device_scan<SumOp, false>(row_units.as<int>(), n_long, dslot.as<int>(),
                                             dslot.as<int>() + n_long, sums.as<int>(), s)))
             return rc;
@@ -781,6 +917,7 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         plan_totals_kernel<<<dim3(1), dim3(128), 0, s>>>(grp_units.as<int>(), (int)n_long,
                                                        totals.as<int>());
         ACCEL_HIP(hipMemcpyAsync(tot, totals.p, sizeof(tot), hipMemcpyDeviceToHost, s));
+        ACCEL_HIP(hipMemcpyAsync(long_cost, qload.p, sizeof(long_cost), hipMemcpyDeviceToHost, s));
     } else {
         ACCEL_HIP(hipMemsetAsync(dslot.p, 0, sizeof(int), s));
     }
@@ -797,14 +934,11 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
             return rc;
         ACCEL_HIP(hipMemcpyAsync(&n_short_units32, scnt.as<int>() + n_short, sizeof(int),
                                  hipMemcpyDeviceToHost, s));
-        ACCEL_HIP(hipStreamSynchronize(s));
-    } else {
-        ACCEL_HIP(hipStreamSynchronize(s));
     }
+    ACCEL_HIP(hipStreamSynchronize(s));
     const int64_t n_short_units = n_short_units32;
     PlanParams pp;
     BinOffsets bo;
-    int64_t longest = 0;
     for (int q = 0; q < kXcds; q++) pp.queue_long[q] = 0;
     for (int b = 0; b < kPlanBins; b++) bo.off[b] = 0;
     if (n_long > 0)
@@ -816,49 +950,86 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
                 bo.off[b] = pp.queue_long[g % kXcds];
                 pp.queue_long[g % kXcds] += tot[b + 1] - tot[b];
             }
-    for (int q = 0; q < kXcds; q++) longest = std::max<int64_t>(longest, pp.queue_long[q]);
     const int64_t n_long_units = n_long > 0 ? tot[kPlanBins] : 0;
-    const int64_t total = n_long_units + n_short_units;
-    int64_t per_queue = std::max(longest, (total + kXcds - 1) / kXcds);
-    per_queue = (per_queue + kWavesPerGroup - 1) / kWavesPerGroup * kWavesPerGroup;
-    // quotas: fill the queues level, shortest first, until the short entries are used up
-    {
-        int64_t left = n_short_units;
-        for (int g = 0; g < kXcds; g++) pp.quota[g] = 0;
-        // raise a common fill level: queue g takes max(0, level - queue_long[g])
-        int64_t lo = 0, hi = per_queue;
+
+    // whole-row units: list them, order them by the caller's row id, cut the sequence into
+    // one share per queue so that long pieces + share cost about the same everywhere
+    DevBuf units(tmp), key(tmp), cost(tmp), heavy(tmp), csums(tmp), first(tmp);
+    uint32_t *order = nullptr;
+    QueueCuts qc;
+    int first_h[kXcds + 1];
+    for (int q = 0; q <= kXcds; q++) { qc.cut[q] = 0; first_h[q] = 0; }
+    if (n_short_units > 0) {
+        const int n = (int)n_short_units;
+        uint32_t *sorted_key = nullptr;
+        if ((rc = units.alloc(sizeof(int4) * (size_t)n))) return rc;
+        if ((rc = key.alloc(sizeof(uint32_t) * (size_t)n))) return rc;
+        if ((rc = cost.alloc(sizeof(int) * (size_t)(n + 1)))) return rc;
+        if ((rc = heavy.alloc(sizeof(int) * (size_t)(n + 1)))) return rc;
+        if ((rc = csums.alloc(sizeof(int) * (size_t)(n / kTile + 4)))) return rc;
+        if ((rc = first.alloc(sizeof(int) * (kXcds + 1)))) return rc;
+        list_short_units_kernel<<<dim3(grid_for(n_short)), dim3(kThreads), 0, s>>>(
+            reinterpret_cast<const int4 *>(h->block4), (int)n_short, unit_nz, scnt.as<int>(), perm,
+            units.as<int4>(), key.as<uint32_t>());
+        if ((rc = radix_sort_pairs(tmp, key.as<uint32_t>(), n, (uint32_t)std::max<int64_t>(h->rows - 1, 0), s,
+                                   &sorted_key, &order)))
+            return rc;
+        const int light_nz = std::max(24, unit_nz / 4);        // a unit up to this size is a light one
+        short_unit_cost_kernel<<<dim3(grid_for(n)), dim3(kThreads), 0, s>>>(
+            units.as<int4>(), order, n, cost_shift, light_nz, cost.as<int>(), heavy.as<int>());
+        if ((rc = device_scan<SumOp, false>(cost.as<int>(), n, cost.as<int>(), cost.as<int>() + n,
+                                            csums.as<int>(), s)))
+            return rc;
+        if ((rc = device_scan<SumOp, false>(heavy.as<int>(), n, heavy.as<int>(), heavy.as<int>() + n,
+                                            csums.as<int>(), s)))
+            return rc;
+        int short_cost = 0;
+        ACCEL_HIP(hipMemcpyAsync(&short_cost, cost.as<int>() + n, sizeof(int), hipMemcpyDeviceToHost, s));
+        ACCEL_HIP(hipStreamSynchronize(s));
+        // raise a common level: queue q takes max(0, level - long_cost[q]) of the short cost
+        int64_t lo = 0, hi = (int64_t)short_cost;
+        for (int q = 0; q < kXcds; q++) hi = std::max<int64_t>(hi, (int64_t)long_cost[q] + short_cost);
         auto taken = [&](int64_t level) {
             int64_t t = 0;
-            for (int g = 0; g < kXcds; g++) t += std::max<int64_t>(0, level - pp.queue_long[g]);
+            for (int q = 0; q < kXcds; q++) t += std::max<int64_t>(0, level - long_cost[q]);
             return t;
         };
-        while (lo < hi) {                              // largest level with taken(level) <= units
-            const int64_t mid = (lo + hi + 1) / 2;
-            if (taken(mid) <= n_short_units) lo = mid; else hi = mid - 1;
+        while (lo < hi) {                              // smallest level that takes all of it
+            const int64_t mid = (lo + hi) / 2;
+            if (taken(mid) >= short_cost) hi = mid; else lo = mid + 1;
         }
-        for (int g = 0; g < kXcds; g++) {
-            pp.quota[g] = (int)std::max<int64_t>(0, lo - pp.queue_long[g]);
-            left -= pp.quota[g];
+        int64_t run = 0;
+        for (int q = 0; q < kXcds; q++) {
+            qc.cut[q] = (int)std::min<int64_t>(run, short_cost);
+            run += std::max<int64_t>(0, lo - long_cost[q]);
         }
-        for (int g = 0; g < kXcds && left > 0; g++)    // remainder: one more for the first queues with room
-            if (pp.queue_long[g] + pp.quota[g] < per_queue) { pp.quota[g]++; left--; }
-        if (left != 0) {
-            set_error("internal: launch plan could not place %lld units", (long long)left);
-            return ACCEL_ERR_ARG;
-        }
+        qc.cut[kXcds] = INT_MAX;
+        if ((rc = fill_u32(first.p, (uint32_t)n, kXcds + 1, s))) return rc;
+        queue_first_kernel<<<dim3(grid_for(n)), dim3(kThreads), 0, s>>>(cost.as<int>(), n, qc,
+                                                                       first.as<int>());
+        ACCEL_HIP(hipMemcpyAsync(first_h, first.p, sizeof(first_h), hipMemcpyDeviceToHost, s));
+        ACCEL_HIP(hipStreamSynchronize(s));
     }
+    int64_t per_queue = 0;
+    for (int q = 0; q < kXcds; q++)
+        per_queue = std::max<int64_t>(per_queue, (int64_t)pp.queue_long[q] + (first_h[q + 1] - first_h[q]));
+    per_queue = (per_queue + kWavesPerGroup - 1) / kWavesPerGroup * kWavesPerGroup;
     const int64_t n_units = per_queue * kXcds;
+    if (n_units > (int64_t)INT_MAX) {
+        set_error("the launch plan would exceed 2^31 work units");
+        return ACCEL_ERR_ARG;
+    }
     DevBuf dwork;
     if ((rc = dwork.alloc(sizeof(int4) * (size_t)n_units))) return rc;
     if (n_units > 0 && (rc = fill_u32(dwork.p, 0u, (size_t)n_units * 4, s))) return rc;
     if (n_long > 0)
         emit_long_units_kernel<<<dim3(grid_for(n_long * kMaxGroups)), dim3(kThreads), 0, s>>>(
             gcount, s_indptr, first_long, dslot.as<int>(), grp_units.as<int>(), (int)n_long, forced,
-            piece_nz, bo, dwork.as<int4>());
-    if (n_short > 0)
-        emit_short_units_kernel<<<dim3(grid_for(n_short)), dim3(kThreads), 0, s>>>(
-            reinterpret_cast<const int4 *>(h->block4), (int)n_short, unit_nz, scnt.as<int>(), pp,
-            dwork.as<int4>());
+            piece_nz, lrank.as<int>(), bo, dwork.as<int4>());
+    if (n_short_units > 0)
+        place_short_units_kernel<<<dim3(grid_for(n_short_units)), dim3(kThreads), 0, s>>>(
+            units.as<int4>(), order, cost.as<int>(), heavy.as<int>(), (int)n_short_units, qc,
+            first.as<int>(), pp, dwork.as<int4>());
     ACCEL_HIP(hipGetLastError());
     ACCEL_HIP(hipStreamSynchronize(s));
     h->n_units = n_units;
@@ -978,35 +1149,12 @@ int preprocess_device(accel_handle *h)
     h->identity_perm = !hs.unsorted;
 
     // ---- degree sort ------------------------------------------------------
-    DevBuf keys_b(&tmp), vals_a(&tmp), vals_b(&tmp), hist(&tmp), sums(&tmp);
     uint32_t *sdeg = deg.as<uint32_t>();
     uint32_t *perm = nullptr;
     if (!h->identity_perm) {
-        const int64_t tiles = (rows + kTile - 1) / kTile;
-        if ((rc = keys_b.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
-        if ((rc = vals_a.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
-        if ((rc = vals_b.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
-        if ((rc = hist.alloc(sizeof(int) * (size_t)(256 * tiles)))) return rc;
-        if ((rc = sums.alloc(sizeof(int) * (size_t)(256 * tiles / kTile + 4)))) return rc;
-        int bits = 0;
-        while (bits < 32 && (hs.max_degree >> bits) != 0) bits++;
-        uint32_t *kin = deg.as<uint32_t>(), *kout = keys_b.as<uint32_t>();
-        uint32_t *vin = nullptr, *vout = vals_a.as<uint32_t>();
-        for (int shift = 0; shift < bits; shift += 8) {
-            radix_hist<<<dim3((unsigned)tiles), dim3(kThreads), 0, s>>>(kin, rows, shift,
-                                                                       hist.as<int>(), tiles);
-            if ((rc = device_scan<SumOp, false>(hist.as<int>(), 256 * tiles, hist.as<int>(),
-                                                nullptr, sums.as<int>(), s)))
-                return rc;
-            radix_scatter<<<dim3((unsigned)tiles), dim3(kThreads), 0, s>>>(
-                kin, vin, kout, vout, rows, shift, hist.as<int>(), tiles);
-            std::swap(kin, kout);
-            vin = vout;
-            vout = (vout == vals_a.as<uint32_t>()) ? vals_b.as<uint32_t>() : vals_a.as<uint32_t>();
-        }
-        ACCEL_HIP(hipGetLastError());
-        sdeg = kin;
-        perm = vin;   // non-null: unsorted input has max_degree >= 1, so at least one pass ran
+        // unsorted input has max_degree >= 1, so at least one pass runs
+        if ((rc = radix_sort_pairs(&tmp, deg.as<uint32_t>(), rows, (uint32_t)hs.max_degree, s, &sdeg, &perm)))
+            return rc;
     }
 
     // ---- sorted indptr ------------------------------------------------------
@@ -1074,7 +1222,7 @@ int preprocess_device(accel_handle *h)
     }
 
     // ---- work list ------------------------------------------------------------
-    if ((rc = build_work_list(&tmp, h, gcount.as<int>(), sip.as<int32_t>(), first_long, n_short_entries, s)))
+    if ((rc = build_work_list(&tmp, h, gcount.as<int>(), sip.as<int32_t>(), first_long, n_short_entries, perm, s)))
         return rc;
 
     h->s_indptr = static_cast<int32_t *>(sip.release());

@@ -167,7 +167,12 @@ int accel_get_sorted_csr(const accel_handle *h, int32_t *indptr, int32_t *idx, f
  * x - 385, sorted row y, first non-zero z, length w <= 384.  w == 0: padding.
  * Workgroup i runs on die i % 8, so units 4*i .. 4*i+3 belong to queue i % 8;
  * the pieces of split rows in queue g only hold columns c with (c >> 3) & 7 == g,
- * ordered by column group ((c >> 3) & (groups - 1)) when there are more than 8.
+ * ordered by column group ((c >> 3) & (groups - 1)) when there are more than 8, and
+ * inside a group by the caller's row id.  Behind them a queue holds its share of the
+ * whole-row units: those are ordered by the caller's row id of their first row, and
+ * that order is cut into eight consecutive shares of about equal load, so that a die
+ * works on a narrow band of the caller's rows at any time (inside a queue the units
+ * of many non-zeros come first, the light ones last).
  * Writes up to cap_units quadruples to out (may be NULL) and the count to *n_units. */
 int accel_get_plan(const accel_handle *h, int32_t *out, int64_t cap_units, int64_t *n_units);
 

@@ -226,18 +226,53 @@ def check_plan(op, n_cols):
         groups = po.row_groups(int(deg[y]), op.info.plan_groups)
         fine = po.column_group(six[z:z + w], groups)
         assert np.all(fine == fine[0]) and fine[0] % 8 == queue[e]   # one group, on its die
-        # a die takes the rows with the most groups first, and its groups in turn
-        key = (-groups, int(fine[0]))
-        assert key >= last.get(queue[e], (-65, 0))
+        # a die takes the rows with the most groups first, its groups in turn, and inside a
+        # group the rows in the order of the caller's row ids
+        key = (-groups, int(fine[0]), int(op.perm()[y]))
+        assert key >= last.get(queue[e], (-65, 0, 0))
         last[queue[e]] = key
     # partial-sum slots: 0 .. n-1, each once, contiguous per row in row order
     slots = long_[:, 0] - 385
     assert sorted(slots.tolist()) == list(range(len(long_)))
     order = np.argsort(slots)
     assert np.all(np.diff(long_[order, 1]) >= 0)
-    per_queue = [int((plan[queue == q][:, 3] != 0).sum()) for q in range(8)]
-    if len(long_) == 0:
-        assert max(per_queue) - min(per_queue) <= 1               # queues are level
+    # whole-row units: behind the pieces in every queue, the eight queues taking consecutive
+    # shares of the order of the caller's row ids (of each unit's first row); inside a queue
+    # the heavy units come first and the light ones last, each kind in that order
+    perm = op.perm()
+    light_nz = max(24, unit // 4)
+    keys = []
+    for q in range(8):
+        mine = plan[queue == q]
+        mine = mine[mine[:, 3] != 0]
+        is_short = mine[:, 0] <= 384
+        n_pieces = int((~is_short).sum())
+        assert not is_short[:n_pieces].any() and is_short[n_pieces:].all()
+        mine = mine[n_pieces:]
+        heavy = mine[:, 0] * (mine[:, 3] & 0xFFFF) > light_nz
+        n_heavy = int(heavy.sum())
+        assert heavy[:n_heavy].all() and not heavy[n_heavy:].any()
+        k = perm[mine[:, 1]]
+        assert np.all(np.diff(k[:n_heavy]) > 0) and np.all(np.diff(k[n_heavy:]) > 0)
+        keys.append(k)
+    for q in range(7):                                  # queue q's rows all precede queue q + 1's
+        later = np.concatenate(keys[q + 1:])
+        if keys[q].size and later.size:
+            assert keys[q].max() < later.min()
+    # ... and the shares level the load: cost = non-zeros + rows + 8 per unit, + 8 per piece
+    load = np.zeros(8)
+    for e in np.flatnonzero(plan[:, 3] != 0):
+        x, y, z, w = plan[e]
+        load[queue[e]] += (w + 9) if x > 384 else (x + 1) * (w & 0xFFFF) + 8
+    heaviest_unit = 384 + 64 + 8
+    short_load = np.array([sum((d + 1) * (i & 0xFFFF) + 8 for d, r, l, i in plan[queue == q] if 0 < d <= 384 and i)
+                           for q in range(8)])
+    with_short = short_load > 0
+    if with_short.sum() > 1:
+        # queues that received whole-row units end up within a few units of each other
+        assert load[with_short].max() - load[with_short].min() <= 8 * heaviest_unit + 0.02 * load.max()
+        # and none of them is lighter than a queue that holds pieces only
+        assert load[~with_short].min(initial=np.inf) >= load[with_short].min() - 8 * heaviest_unit
 
 
 @pytest.mark.parametrize("team", [1, 2])
