@@ -595,14 +595,29 @@ __device__ __forceinline__ int64_t plan_index(int queue, int pos)
     return ((int64_t)(pos / kWavesPerGroup) * kXcds + queue) * kWavesPerGroup + pos % kWavesPerGroup;
 }
 
-// The split rows in the order of the caller's row ids: key[lr] = that id, and, after the
-// sort, rank[order[i]] = i.
+// The order of the split rows inside their (class, group) bins: key[lr] = the caller's row id
+// (or, for the longest rows, a key that puts the largest first), and, after the sort,
+// rank[order[i]] = i.  Only the order among rows of one class matters.
+// Rows stored in up to this many column groups follow the caller's row ids inside their
+// bins; the longer ones keep "largest first" (they touch all of X whatever their id, and the
+// hub workload measured 2 % faster that way: 2.31 against 2.36 ms at N = 256).
+#ifndef ACCEL_ID_ORDER_MAX_GROUPS
+#define ACCEL_ID_ORDER_MAX_GROUPS 8
+#endif
 __global__ __launch_bounds__(kThreads) void long_row_key_kernel(const uint32_t *__restrict__ perm,
+                                                                const int32_t *__restrict__ s_indptr,
+                                                                int forced_groups,
                                                                 int64_t first_long, int n_long,
                                                                 uint32_t *__restrict__ key)
 {
     const int lr = blockIdx.x * kThreads + threadIdx.x;
-    if (lr < n_long) key[lr] = perm ? perm[first_long + lr] : (uint32_t)(first_long + lr);
+    if (lr >= n_long) return;
+    const int64_t row = first_long + lr;
+    const int ng = row_groups(s_indptr[row + 1] - s_indptr[row], forced_groups);
+    if (ng <= ACCEL_ID_ORDER_MAX_GROUPS)
+        key[lr] = perm ? perm[row] : (uint32_t)row;
+    else
+        key[lr] = (uint32_t)(n_long - 1 - lr);          // largest rows first
 }
 
 __global__ __launch_bounds__(kThreads) void invert_order_kernel(const uint32_t *__restrict__ order, int n,
@@ -853,9 +868,9 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
 // Workgroups are dispatched to the eight dies round-robin (workgroup i runs on
 // die i % 8), so the list is laid out as eight interleaved queues.  Column group
 // g belongs to die g % 8.  A queue holds, in this order: the pieces of the rows
-// stored in 64 groups (the longest rows), one group after the other, the rows of
-// a group in the order of the caller's row ids; then the same for the rows with
-// 32, 16 and 8 groups; then the
+// stored in 64 groups (the longest rows), one group after the other, largest
+// rows first; then the same for the rows with 32, 16 and 8 groups (the rows of
+// an 8-group bin in the order of the caller's row ids); then the
 // queue's share of the whole-row units.  While a die works through one group its
 // L2 only has to hold that group's share of X.
 // The whole-row units are put in the order of the caller's row ids (of each unit's
@@ -891,13 +906,13 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         if ((rc = qload.alloc(sizeof(int) * kXcds))) return rc;
         if ((rc = fill_u32(grp_units.p, 0u, (size_t)n_bins + 1, s))) return rc;
         if ((rc = fill_u32(qload.p, 0u, kXcds, s))) return rc;
-        // inside a (row class, column group) bin the rows follow the caller's row ids, like the
-        // whole-row units further down
+        // inside an 8-group bin the rows follow the caller's row ids, like the whole-row units
+        // further down
         uint32_t *lkey_sorted = nullptr, *lorder = nullptr;
         if ((rc = lkey.alloc(sizeof(uint32_t) * (size_t)n_long))) return rc;
         if ((rc = lrank.alloc(sizeof(int) * (size_t)n_long))) return rc;
-        long_row_key_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(perm, first_long, (int)n_long,
-                                                                             lkey.as<uint32_t>());
+        long_row_key_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(
+            perm, s_indptr, forced, first_long, (int)n_long, lkey.as<uint32_t>());
         if ((rc = radix_sort_pairs(tmp, lkey.as<uint32_t>(), n_long, (uint32_t)std::max<int64_t>(h->rows - 1, 0),
                                    s, &lkey_sorted, &lorder)))
             return rc;

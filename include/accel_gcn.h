@@ -168,7 +168,8 @@ int accel_get_sorted_csr(const accel_handle *h, int32_t *indptr, int32_t *idx, f
  * Workgroup i runs on die i % 8, so units 4*i .. 4*i+3 belong to queue i % 8;
  * the pieces of split rows in queue g only hold columns c with (c >> 3) & 7 == g,
  * ordered by column group ((c >> 3) & (groups - 1)) when there are more than 8, and
- * inside a group by the caller's row id.  Behind them a queue holds its share of the
+ * inside a group by the caller's row id (rows of 8 groups; longer rows: largest
+ * first).  Behind them a queue holds its share of the
  * whole-row units: those are ordered by the caller's row id of their first row, and
  * that order is cut into eight consecutive shares of about equal load, so that a die
  * works on a narrow band of the caller's rows at any time (inside a queue the units

@@ -226,10 +226,10 @@ def check_plan(op, n_cols):
         groups = po.row_groups(int(deg[y]), op.info.plan_groups)
         fine = po.column_group(six[z:z + w], groups)
         assert np.all(fine == fine[0]) and fine[0] % 8 == queue[e]   # one group, on its die
-        # a die takes the rows with the most groups first, its groups in turn, and inside a
-        # group the rows in the order of the caller's row ids
-        key = (-groups, int(fine[0]), int(op.perm()[y]))
-        assert key >= last.get(queue[e], (-65, 0, 0))
+        # a die takes the rows with the most groups first and its groups in turn; inside a group
+        # the rows follow the caller's row ids (8-group rows) or come largest first (longer rows)
+        key = (-groups, int(fine[0]), int(op.perm()[y]) if groups == 8 else -int(y))
+        assert key >= last.get(queue[e], (-65, 0, -2 ** 40))
         last[queue[e]] = key
     # partial-sum slots: 0 .. n-1, each once, contiguous per row in row order
     slots = long_[:, 0] - 385
