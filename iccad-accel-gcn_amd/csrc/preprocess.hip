@@ -774,9 +774,15 @@ __global__ __launch_bounds__(kThreads) void queue_first_kernel(const int *__rest
     for (int i = q_prev + 1; i <= q; i++) first[i] = sidx;
 }
 
-// Inside its queue a unit goes behind the pieces; the units with many non-zeros first, the
-// light ones last (both in the order of the caller's row ids), so that a queue does not end
-// on a long chain of gathers.  heavy_before[s] = heavy units among the first s, [n] = all.
+// Inside its queue a unit goes behind the pieces, in the order of the caller's row ids,
+// except that the queue's last kTailLight light units (few non-zeros: short chains of
+// gathers) are held back and placed at the very end, so that a queue does not end on a
+// long chain.  They are the light units with the highest ids of the queue's share, i.e.
+// they lie in the band of rows the die is working on at that time anyway.
+// heavy_before[s] = heavy units among the first s, [n] = all.
+#ifndef ACCEL_TAIL_LIGHT
+#define ACCEL_TAIL_LIGHT 2048                // two rounds of the 1,024 wavefronts a die holds
+#endif
 __global__ __launch_bounds__(kThreads) void place_short_units_kernel(
     const int4 *__restrict__ units, const uint32_t *__restrict__ order, const int *__restrict__ running,
     const int *__restrict__ heavy_before, int n, QueueCuts qc, const int *__restrict__ first,
@@ -785,11 +791,17 @@ __global__ __launch_bounds__(kThreads) void place_short_units_kernel(
     const int sidx = blockIdx.x * kThreads + threadIdx.x;
     if (sidx >= n) return;
     const int q = queue_of(running[sidx], qc);
-    const int f = first[q], f_next = first[q + 1];
-    const int h0 = heavy_before[f], h_all = heavy_before[f_next] - h0;     // heavy units of this queue
-    const int h_me = heavy_before[sidx] - h0;                              // ... before this unit
-    const bool is_heavy = heavy_before[sidx + 1] != heavy_before[sidx];
-    const int pos = is_heavy ? h_me : h_all + (sidx - f) - h_me;
+    const int f = first[q], n_q = first[q + 1] - f;
+    const int h0 = heavy_before[f];
+    const int light_all = n_q - (heavy_before[f + n_q] - h0);              // light units of this queue
+    const int light_me = (sidx - f) - (heavy_before[sidx] - h0);           // ... before this unit
+    const bool is_light = heavy_before[sidx + 1] == heavy_before[sidx];
+    const int kept = max(0, light_all - ACCEL_TAIL_LIGHT);                 // light units that stay in line
+    int pos;
+    if (is_light && light_me >= kept)
+        pos = n_q - (light_all - light_me);                                // held back: the last ones
+    else
+        pos = (sidx - f) - max(0, light_me - kept);                        // in line, minus those held back before it
     work[plan_index(q, pp.queue_long[q] + pos)] = units[order[sidx]];
 }
 

@@ -172,8 +172,8 @@ int accel_get_sorted_csr(const accel_handle *h, int32_t *indptr, int32_t *idx, f
  * first).  Behind them a queue holds its share of the
  * whole-row units: those are ordered by the caller's row id of their first row, and
  * that order is cut into eight consecutive shares of about equal load, so that a die
- * works on a narrow band of the caller's rows at any time (inside a queue the units
- * of many non-zeros come first, the light ones last).
+ * works on a narrow band of the caller's rows at any time (the last 2048 units of
+ * few non-zeros of a share are held back to the end of their queue).
  * Writes up to cap_units quadruples to out (may be NULL) and the count to *n_units. */
 int accel_get_plan(const accel_handle *h, int32_t *out, int64_t cap_units, int64_t *n_units);
 

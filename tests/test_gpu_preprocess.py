@@ -238,7 +238,8 @@ def check_plan(op, n_cols):
     assert np.all(np.diff(long_[order, 1]) >= 0)
     # whole-row units: behind the pieces in every queue, the eight queues taking consecutive
     # shares of the order of the caller's row ids (of each unit's first row); inside a queue
-    # the heavy units come first and the light ones last, each kind in that order
+    # they keep that order, except that the last 2,048 light units of the share (all of them
+    # if there are fewer) are held back to the very end
     perm = op.perm()
     light_nz = max(24, unit // 4)
     keys = []
@@ -249,11 +250,14 @@ def check_plan(op, n_cols):
         n_pieces = int((~is_short).sum())
         assert not is_short[:n_pieces].any() and is_short[n_pieces:].all()
         mine = mine[n_pieces:]
-        heavy = mine[:, 0] * (mine[:, 3] & 0xFFFF) > light_nz
-        n_heavy = int(heavy.sum())
-        assert heavy[:n_heavy].all() and not heavy[n_heavy:].any()
         k = perm[mine[:, 1]]
-        assert np.all(np.diff(k[:n_heavy]) > 0) and np.all(np.diff(k[n_heavy:]) > 0)
+        light = mine[:, 0] * (mine[:, 3] & 0xFFFF) <= light_nz
+        n_tail = min(2048, int(light.sum()))
+        in_line = len(k) - n_tail
+        assert light[in_line:].all()
+        assert np.all(np.diff(k[:in_line]) > 0) and np.all(np.diff(k[in_line:]) > 0)
+        if n_tail and light[:in_line].any():             # held back: the light units with the highest ids
+            assert k[in_line:].min() > k[:in_line][light[:in_line]].max()
         keys.append(k)
     for q in range(7):                                  # queue q's rows all precede queue q + 1's
         later = np.concatenate(keys[q + 1:])
