@@ -606,7 +606,7 @@ __device__ __forceinline__ int64_t plan_index(int queue, int pos)
 #endif
 __global__ __launch_bounds__(kThreads) void long_row_key_kernel(const uint32_t *__restrict__ perm,
                                                                 const int32_t *__restrict__ s_indptr,
-                                                                int forced_groups,
+                                                                int forced_groups, int key_shift,
                                                                 int64_t first_long, int n_long,
                                                                 uint32_t *__restrict__ key)
 {
@@ -615,9 +615,9 @@ __global__ __launch_bounds__(kThreads) void long_row_key_kernel(const uint32_t *
     const int64_t row = first_long + lr;
     const int ng = row_groups(s_indptr[row + 1] - s_indptr[row], forced_groups);
     if (ng <= ACCEL_ID_ORDER_MAX_GROUPS)
-        key[lr] = perm ? perm[row] : (uint32_t)row;
+        key[lr] = (perm ? perm[row] : (uint32_t)row) >> key_shift;
     else
-        key[lr] = (uint32_t)(n_long - 1 - lr);          // largest rows first
+        key[lr] = (uint32_t)(n_long - 1 - lr) >> key_shift;   // largest rows first
 }
 
 __global__ __launch_bounds__(kThreads) void invert_order_kernel(const uint32_t *__restrict__ order, int n,
@@ -707,7 +707,8 @@ __device__ __forceinline__ int unit_cost(int nz, int n_rows, int shift)
 // first row: the key the units are queued by.
 __global__ __launch_bounds__(kThreads) void list_short_units_kernel(
     const int4 *__restrict__ block4, int n_short, int unit_nz, const int *__restrict__ first_unit,
-    const uint32_t *__restrict__ perm, int4 *__restrict__ units, uint32_t *__restrict__ key)
+    const uint32_t *__restrict__ perm, int key_shift, int4 *__restrict__ units,
+    uint32_t *__restrict__ key)
 {
     const int j = blockIdx.x * kThreads + threadIdx.x;
     if (j >= n_short) return;
@@ -716,7 +717,7 @@ __global__ __launch_bounds__(kThreads) void list_short_units_kernel(
     int i = first_unit[j];
     for (int r = 0; r < n_rows; r += rpu, i++) {
         units[i] = make_int4(d, b.y + r, b.z + r * d, (w_nz << 16) + min(rpu, n_rows - r));
-        key[i] = perm ? perm[b.y + r] : (uint32_t)(b.y + r);
+        key[i] = (perm ? perm[b.y + r] : (uint32_t)(b.y + r)) >> key_shift;
     }
 }
 
@@ -733,22 +734,26 @@ __global__ __launch_bounds__(kThreads) void short_unit_cost_kernel(
 }
 
 // Non-zeros and pieces of the split rows per queue (column group g belongs to queue g % 8).
+// Thread t looks at (row t / 64, group t % 64), so lane l of a wavefront always holds a
+// group of queue l % 8: the wavefront's eight sums are formed with shuffles.
 __global__ __launch_bounds__(kThreads) void long_queue_load_kernel(
     const int *__restrict__ gcount, int n_long, int piece, int shift, int *__restrict__ queue_cost)
 {
-    __shared__ int part[kXcds];
-    if (threadIdx.x < kXcds) part[threadIdx.x] = 0;
-    __syncthreads();
-    const int64_t t = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    if (t < (int64_t)n_long * kMaxGroups) {
+    static_assert(kMaxGroups == 64, "one wavefront per split row");
+    const int64_t n = (int64_t)n_long * kMaxGroups;
+    int v = 0;                                           // the stride keeps t % 64 == lane
+    for (int64_t t = (int64_t)blockIdx.x * kThreads + threadIdx.x; t < n; t += (int64_t)gridDim.x * kThreads) {
         const int c = gcount[t];
         if (c > 0) {
             const int pieces = (c + piece - 1) / piece;
-            atomicAdd(&part[(int)(t % kMaxGroups) % kXcds], ((c + 9 * pieces) >> shift) + pieces);
+            v += ((c + 9 * pieces) >> shift) + pieces;
         }
     }
-    __syncthreads();
-    if (threadIdx.x < kXcds && part[threadIdx.x]) atomicAdd(&queue_cost[threadIdx.x], part[threadIdx.x]);
+    v += __shfl_xor(v, 8);
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    const int lane = threadIdx.x & 63;
+    if (lane < kXcds && v) atomicAdd(&queue_cost[lane], v);
 }
 
 struct QueueCuts {
@@ -906,6 +911,11 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
     int rc;
     int tot[kPlanBins + 1] = {0};
     int long_cost[kXcds] = {0};
+    // the order by row id is kept to 16 bits (two passes of the sort): bands of rows, not single
+    // rows, are what the caches see; equal keys stay in row order (the sort is stable)
+    int key_shift = 0;
+    while ((std::max<int64_t>(h->rows, 1) - 1) >> key_shift >= 65536) key_shift++;
+    const uint32_t max_key = (uint32_t)((std::max<int64_t>(h->rows, 1) - 1) >> key_shift);
     int cost_shift = 2;                                // total cost = about (nnz + 10 rows) >> shift + units < 2^31
     while ((((int64_t)h->nnz + 10 * h->rows) >> cost_shift) + h->rows >= ((int64_t)1 << 30)) cost_shift++;
     if ((rc = dslot.alloc(sizeof(int) * (size_t)(n_long + 1)))) return rc;
@@ -924,16 +934,15 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         if ((rc = lkey.alloc(sizeof(uint32_t) * (size_t)n_long))) return rc;
         if ((rc = lrank.alloc(sizeof(int) * (size_t)n_long))) return rc;
         long_row_key_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(
-            perm, s_indptr, forced, first_long, (int)n_long, lkey.as<uint32_t>());
-        if ((rc = radix_sort_pairs(tmp, lkey.as<uint32_t>(), n_long, (uint32_t)std::max<int64_t>(h->rows - 1, 0),
-                                   s, &lkey_sorted, &lorder)))
+            perm, s_indptr, forced, key_shift, first_long, (int)n_long, lkey.as<uint32_t>());
+        if ((rc = radix_sort_pairs(tmp, lkey.as<uint32_t>(), n_long, max_key, s, &lkey_sorted, &lorder)))
             return rc;
         invert_order_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(lorder, (int)n_long,
                                                                              lrank.as<int>());
         long_unit_count_kernel<<<dim3(grid_for(n_long)), dim3(kThreads), 0, s>>>(
             gcount, s_indptr, first_long, (int)n_long, forced, piece_nz, lrank.as<int>(),
             row_units.as<int>(), grp_units.as<int>());
-        long_queue_load_kernel<<<dim3(grid_for(n_long * kMaxGroups)), dim3(kThreads), 0, s>>>(
+        long_queue_load_kernel<<<dim3(std::min(grid_for(n_long * kMaxGroups), 1024u)), dim3(kThreads), 0, s>>>(
             gcount, (int)n_long, piece_nz, cost_shift, qload.as<int>());
         if ((rc = device_scan<SumOp, false>(row_units.as<int>(), n_long, dslot.as<int>(),
                                             dslot.as<int>() + n_long, sums.as<int>(), s)))
@@ -997,9 +1006,8 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         if ((rc = first.alloc(sizeof(int) * (kXcds + 1)))) return rc;
         list_short_units_kernel<<<dim3(grid_for(n_short)), dim3(kThreads), 0, s>>>(
             reinterpret_cast<const int4 *>(h->block4), (int)n_short, unit_nz, scnt.as<int>(), perm,
-            units.as<int4>(), key.as<uint32_t>());
-        if ((rc = radix_sort_pairs(tmp, key.as<uint32_t>(), n, (uint32_t)std::max<int64_t>(h->rows - 1, 0), s,
-                                   &sorted_key, &order)))
+            key_shift, units.as<int4>(), key.as<uint32_t>());
+        if ((rc = radix_sort_pairs(tmp, key.as<uint32_t>(), n, max_key, s, &sorted_key, &order)))
             return rc;
         const int light_nz = std::max(24, unit_nz / 4);        // a unit up to this size is a light one
         short_unit_cost_kernel<<<dim3(grid_for(n)), dim3(kThreads), 0, s>>>(

@@ -220,6 +220,11 @@ def check_plan(op, n_cols):
     assert np.all(covered == 1)
     # queue of unit e is (e // 4) % 8
     queue = (np.arange(plan.shape[0]) // 4) % 8
+    # the plan orders by the caller's row id in bands: the id's top 16 bits
+    shift = 0
+    while (max(deg.size, 1) - 1) >> shift >= 65536:
+        shift += 1
+    n_split = int((deg > split).sum())
     last = {}
     for e in np.flatnonzero((plan[:, 3] != 0) & (plan[:, 0] > 384)):
         x, y, z, w = plan[e]
@@ -228,8 +233,10 @@ def check_plan(op, n_cols):
         assert np.all(fine == fine[0]) and fine[0] % 8 == queue[e]   # one group, on its die
         # a die takes the rows with the most groups first and its groups in turn; inside a group
         # the rows follow the caller's row ids (8-group rows) or come largest first (longer rows)
-        key = (-groups, int(fine[0]), int(op.perm()[y]) if groups == 8 else -int(y))
-        assert key >= last.get(queue[e], (-65, 0, -2 ** 40))
+        key = (-groups, int(fine[0]),
+               int(op.perm()[y]) >> shift if groups == 8 else (deg.size - 1 - int(y)) >> shift)
+        assert deg.size - n_split <= y
+        assert key >= last.get(queue[e], (-65, 0, -1))
         last[queue[e]] = key
     # partial-sum slots: 0 .. n-1, each once, contiguous per row in row order
     slots = long_[:, 0] - 385
@@ -250,19 +257,21 @@ def check_plan(op, n_cols):
         n_pieces = int((~is_short).sum())
         assert not is_short[:n_pieces].any() and is_short[n_pieces:].all()
         mine = mine[n_pieces:]
-        k = perm[mine[:, 1]]
+        k = perm[mine[:, 1]] >> shift
         light = mine[:, 0] * (mine[:, 3] & 0xFFFF) <= light_nz
         n_tail = min(2048, int(light.sum()))
         in_line = len(k) - n_tail
         assert light[in_line:].all()
-        assert np.all(np.diff(k[:in_line]) > 0) and np.all(np.diff(k[in_line:]) > 0)
+        assert np.all(np.diff(k[:in_line]) >= 0) and np.all(np.diff(k[in_line:]) >= 0)
+        if shift == 0:
+            assert np.all(np.diff(k[:in_line]) > 0) and np.all(np.diff(k[in_line:]) > 0)
         if n_tail and light[:in_line].any():             # held back: the light units with the highest ids
-            assert k[in_line:].min() > k[:in_line][light[:in_line]].max()
+            assert k[in_line:].min() >= k[:in_line][light[:in_line]].max()
         keys.append(k)
     for q in range(7):                                  # queue q's rows all precede queue q + 1's
         later = np.concatenate(keys[q + 1:])
         if keys[q].size and later.size:
-            assert keys[q].max() < later.min()
+            assert keys[q].max() <= later.min()
     # ... and the shares level the load: cost = non-zeros + rows + 8 per unit, + 8 per piece
     load = np.zeros(8)
     for e in np.flatnonzero(plan[:, 3] != 0):
@@ -286,6 +295,20 @@ def test_launch_plan(gpu, seed, n_long, team):
     op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_team=team)
     assert (op.info.plan_unit_nz, op.info.plan_split_nz) == ((48, 384) if team == 2 else (48, 48))
     check_plan(op, g.n_cols)
+    op.close()
+
+
+def test_launch_plan_row_bands(gpu):
+    """More than 65,536 rows: the plan orders by bands of row ids (the id's top 16 bits)."""
+    rng = np.random.default_rng(21)
+    deg = rng.integers(0, 9, 140_000)
+    deg[rng.integers(0, deg.size, 40)] = rng.integers(200, 3000, 40)
+    g = helpers.graph_from_degrees(deg, n_cols=5000, seed=21)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_team=1)
+    check_plan(op, g.n_cols)
+    X = rng.uniform(-1, 1, (g.n_cols, 8)).astype(np.float32)
+    from oracle import spmm_oracle as so
+    assert so.check(op.matmul(X), g.indptr, g.indices, g.values, X) <= so.TOL
     op.close()
 
 
