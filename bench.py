@@ -98,6 +98,16 @@ def fixture_graph(pkg, name, seed=0, sigma=0):
     return g
 
 
+def uniform_graph(pkg, n_rows, degree, n_cols, seed=0):
+    """Every row has `degree` non-zeros with columns uniform over n_cols (repeats
+    allowed): a probe of the gather rate for an X of a chosen size."""
+    rng = np.random.default_rng(seed)
+    indptr = (np.arange(n_rows + 1, dtype=np.int64) * degree).astype(np.int32)
+    indices = rng.integers(0, n_cols, size=n_rows * degree).astype(np.int32)
+    values = rng.random(n_rows * degree, dtype=np.float32)
+    return pkg.synthetic.Graph(f"uniform:{n_rows}:{degree}:{n_cols}", indptr, indices, values, n_rows, n_cols)
+
+
 def rocsparse_baseline(pkg, op, g, dX, N, iters=10):
     """Vendor-library CSR SpMM on the same resident operands (comparison only, as
     upstream compares with cuSPARSE; never part of `value`)."""
@@ -161,7 +171,8 @@ def main():
                     help="cfg1..cfg5, or fixture:<name> for the degree sequence of one of the "
                          "reference's graphs (e.g. fixture:OVCAR-8H, fixture:ppa) with uniform random "
                          "columns, or local:<name>:<sigma> for the same with columns within about "
-                         "sigma of the row id")
+                         "sigma of the row id, or uniform:<rows>:<degree>:<cols> for rows of one "
+                         "degree with uniform random columns")
     ap.add_argument("--N", type=int, default=0, help="columns of X (default: the workload's first)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the scipy baseline and the check")
     ap.add_argument("--compare-rocsparse", action="store_true",
@@ -198,6 +209,9 @@ def main():
     t0 = time.time()
     if a.workload.startswith("fixture:"):
         g = fixture_graph(pkg, a.workload.split(":", 1)[1])
+    elif a.workload.startswith("uniform:"):             # uniform:<rows>:<degree>:<cols>
+        _, n_rows, degree, n_cols = a.workload.split(":")
+        g = uniform_graph(pkg, int(n_rows), int(degree), int(n_cols))
     elif a.workload.startswith("local:"):               # local:<name>:<sigma>
         _, name, sigma = a.workload.split(":")
         g = fixture_graph(pkg, name, sigma=int(sigma))
