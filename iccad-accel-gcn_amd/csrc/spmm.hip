@@ -54,6 +54,12 @@ __host__ __device__ inline int zero_rows_per_group(int N) { return N >= kZeroFlo
 #ifndef ACCEL_TEAM_UNROLL
 #define ACCEL_TEAM_UNROLL 4               // the same for the kernel with workgroup units (8: 5-10 % slower)
 #endif
+#ifndef ACCEL_STREAMING_STORES
+#define ACCEL_STREAMING_STORES 1
+#endif
+#ifndef ACCEL_STREAMING_MIN_BYTES
+#define ACCEL_STREAMING_MIN_BYTES 128        // rows shorter than a cache line are stored the ordinary way
+#endif
 constexpr int kUnroll = ACCEL_UNROLL;
 constexpr int kTeamUnroll = ACCEL_TEAM_UNROLL;
 constexpr int kPanel = ACCEL_PANEL;
@@ -85,7 +91,92 @@ __device__ __forceinline__ void store_vec(float *__restrict__ p, const float (&v
     }
 }
 
+// Rows of Y are written once and not read again by this launch: a streaming
+// (non-temporal) store.  Measured on this GPU with gathers that hit L2: one ordinary
+// 256-byte store per 32 gathers lowers the gather rate from 27 to 20 TB/s, a
+// non-temporal one to 26 TB/s.
+template <int VEC>
+__device__ __forceinline__ void store_vec_streaming(float *__restrict__ p, const float (&v)[VEC], bool streaming)
+{
+#if ACCEL_STREAMING_STORES
+    if (!streaming) {
+        store_vec<VEC>(p, v);
+    } else if constexpr (VEC == 4) {
+        typedef float v4f __attribute__((ext_vector_type(4)));
+        const v4f t = {v[0], v[1], v[2], v[3]};
+        __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
+    } else if constexpr (VEC == 2) {
+        typedef float v2f __attribute__((ext_vector_type(2)));
+        const v2f t = {v[0], v[1]};
+        __builtin_nontemporal_store(t, reinterpret_cast<v2f *>(p));
+    } else {
+        __builtin_nontemporal_store(v[0], p);
+    }
+#else
+    store_vec<VEC>(p, v);
+#endif
+}
+
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// One lane group's share of one row: non-zeros k, k + gp, ... of the d pairs at row_st are
+// multiplied with their rows of X and added into acc.  U gathers are issued back to back;
+// full batches carry no masks, only the last batch of a row is predicated.
+// The staged pair holds the value and, when the operand is smaller than 4 GiB (kWide ==
+// false), the byte offset of the row of X, so that the address is one 32-bit add to a
+// uniform base; otherwise the column, and the address is formed with 64-bit arithmetic.
+template <int VEC, int U, bool kWide>
+__device__ __forceinline__ void gather_row(const int2 *__restrict__ row_st, int d, int k, int gp,
+                                           const float *__restrict__ X, int col, int ld,
+                                           float (&acc)[VEC])
+{
+    const char *xb = reinterpret_cast<const char *>(X);
+    const uint32_t lane_off = (uint32_t)col * 4u;
+    auto fetch = [&](int where, float (&x)[VEC]) {
+        if constexpr (kWide)
+            load_vec<VEC>(X + col + (int64_t)where * ld, x);
+        else
+            load_vec<VEC>(reinterpret_cast<const float *>(xb + ((uint32_t)where + lane_off)), x);
+    };
+    int o = k;
+    for (; o + (U - 1) * gp < d; o += U * gp) {          // full batches
+        int2 p[U];
+        float x[U][VEC];
+#pragma unroll
+        for (int u = 0; u < U; u++) p[u] = row_st[o + u * gp];
+#pragma unroll
+        for (int u = 0; u < U; u++) fetch(p[u].x, x[u]);
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const float a = __int_as_float(p[u].y);
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[u][v], acc[v]);
+        }
+    }
+    if (o < d) {                                         // the row's last, partial batch
+        int2 p[U];
+        float x[U][VEC];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int ou = o + u * gp;
+            ok[u] = ou < d;
+            p[u] = row_st[ok[u] ? ou : k];
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int v = 0; v < VEC; v++) x[u][v] = 0.0f;
+            if (ok[u]) fetch(p[u].x, x[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const float a = ok[u] ? __int_as_float(p[u].y) : 0.0f;
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[u][v], acc[v]);
+        }
+    }
+}
 
 // Zero-degree rows are the first n_zero_rows rows of the sorted order; the workgroups at
 // the head of the grid write them (act(bias) with an epilogue).  They come first so that
@@ -107,11 +198,11 @@ __device__ __forceinline__ void zero_fill_rows(const int32_t *__restrict__ perm,
             float t = bias ? bias[c + v] : 0.0f;                // A X is 0 for this row
             fill[v] = relu ? fmaxf(t, 0.0f) : t;
         }
-        store_vec<VEC>(Y + out_row * ld + c, fill);
+        store_vec_streaming<VEC>(Y + out_row * ld + c, fill, N * 4 >= ACCEL_STREAMING_MIN_BYTES);
     }
 }
 
-template <int L, int VEC>
+template <int L, int VEC, bool kWide>
 __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     const int4 *__restrict__ work, int n_units,
     const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
@@ -164,7 +255,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 #pragma unroll
         for (int j = 0; j < kRounds; j++) {
             const int i = lane + 64 * j;
-            if (i < total_nz) st[i] = make_int2(ci[j], __float_as_int(cv[j]));
+            if (i < total_nz) st[i] = make_int2(kWide ? ci[j] : (int)((uint32_t)ci[j] * ((uint32_t)ld * 4u)), __float_as_int(cv[j]));
         }
     }
     __builtin_amdgcn_wave_barrier();
@@ -186,6 +277,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     const int k = g & (gp - 1);          // which of the row's gp groups this is
     const int rloc = g >> lg;            // which of the rows in flight
 
+    const bool streaming = N * 4 >= ACCEL_STREAMING_MIN_BYTES;
     for (int c0 = 0; c0 < N; c0 += CW) {
         const int col = c0 + sub * VEC;
         const bool col_ok = col < N;
@@ -195,35 +287,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
             float acc[VEC];
 #pragma unroll
             for (int v = 0; v < VEC; v++) acc[v] = 0.0f;
-            if (live) {
-                const int2 *row_st = st + r * d;
-                const float *xcol = X + col;
-                // every batch issues up to kUnroll gathers; lanes past the end of the
-                // row are masked, so a row costs ceil(d / (gp * kUnroll)) round trips
-                for (int o = k; o < d; o += kUnroll * gp) {
-                    int2 p[kUnroll];
-                    float x[kUnroll][VEC];
-                    bool ok[kUnroll];
-#pragma unroll
-                    for (int u = 0; u < kUnroll; u++) {
-                        const int ou = o + u * gp;
-                        ok[u] = ou < d;
-                        p[u] = row_st[ok[u] ? ou : k];
-                    }
-#pragma unroll
-                    for (int u = 0; u < kUnroll; u++) {
-#pragma unroll
-                        for (int v = 0; v < VEC; v++) x[u][v] = 0.0f;
-                        if (ok[u]) load_vec<VEC>(xcol + (int64_t)p[u].x * ld, x[u]);
-                    }
-#pragma unroll
-                    for (int u = 0; u < kUnroll; u++) {
-                        const float a = ok[u] ? __int_as_float(p[u].y) : 0.0f;
-#pragma unroll
-                        for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[u][v], acc[v]);
-                    }
-                }
-            }
+            if (live) gather_row<VEC, kUnroll, kWide>(st + r * d, d, k, gp, X, col, ld, acc);
             // add the gp partial sums of each row (all lanes take part)
             for (int m = L; m < (L << lg); m <<= 1) {
 #pragma unroll
@@ -231,9 +295,10 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
             }
             const int64_t out_row = __shfl(my_out, r < n_rows ? r : 0);
             if (live && k == 0) {
-                if (is_long)
-                    store_vec<VEC>(partial + (int64_t)(deg - (kDegBound + 1)) * ld + col, acc);
-                else {
+                if (is_long) {
+                    store_vec_streaming<VEC>(partial + (int64_t)(deg - (kDegBound + 1)) * ld + col, acc,
+                                             streaming);
+                } else {
                     if (bias) {
 #pragma unroll
                         for (int v = 0; v < VEC; v++) acc[v] += bias[col + v];
@@ -242,7 +307,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 #pragma unroll
                         for (int v = 0; v < VEC; v++) acc[v] = fmaxf(acc[v], 0.0f);
                     }
-                    store_vec<VEC>(Y + out_row * ld + col, acc);
+                    store_vec_streaming<VEC>(Y + out_row * ld + col, acc, streaming);
                 }
             }
         }
@@ -254,7 +319,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 // several wavefronts their sums meet in LDS.  Used for small matrices, where the time of
 // a launch is the longest chain of dependent gathers in one wavefront: the chain is four
 // times shorter and rows of up to one unit need no partial sums.
-template <int L, int VEC>
+template <int L, int VEC, bool kWide>
 __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
     const int4 *__restrict__ work, int n_units,
     const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
@@ -302,7 +367,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
 #pragma unroll
         for (int j = 0; j < kRounds; j++) {
             const int i = (int)threadIdx.x + kWgThreads * j;
-            if (i < total_nz) stage[i] = make_int2(ci[j], __float_as_int(cv[j]));
+            if (i < total_nz) stage[i] = make_int2(kWide ? ci[j] : (int)((uint32_t)ci[j] * ((uint32_t)ld * 4u)), __float_as_int(cv[j]));
         }
     }
     __syncthreads();
@@ -336,33 +401,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
             float acc[VEC];
 #pragma unroll
             for (int v = 0; v < VEC; v++) acc[v] = 0.0f;
-            if (live) {
-                const int2 *row_st = stage + r * d;
-                const float *xcol = X + col;
-                for (int o = k; o < d; o += kTeamUnroll * gp) {
-                    int2 p[kTeamUnroll];
-                    float x[kTeamUnroll][VEC];
-                    bool ok[kTeamUnroll];
-#pragma unroll
-                    for (int u = 0; u < kTeamUnroll; u++) {
-                        const int ou = o + u * gp;
-                        ok[u] = ou < d;
-                        p[u] = row_st[ok[u] ? ou : k];
-                    }
-#pragma unroll
-                    for (int u = 0; u < kTeamUnroll; u++) {
-#pragma unroll
-                        for (int v = 0; v < VEC; v++) x[u][v] = 0.0f;
-                        if (ok[u]) load_vec<VEC>(xcol + (int64_t)p[u].x * ld, x[u]);
-                    }
-#pragma unroll
-                    for (int u = 0; u < kTeamUnroll; u++) {
-                        const float a = ok[u] ? __int_as_float(p[u].y) : 0.0f;
-#pragma unroll
-                        for (int v = 0; v < VEC; v++) acc[v] = fmaf(a, x[u][v], acc[v]);
-                    }
-                }
-            }
+            if (live) gather_row<VEC, kTeamUnroll, kWide>(stage + r * d, d, k, gp, X, col, ld, acc);
             // the row's groups inside this wavefront (all lanes take part)
             for (int m = L; m < L * in_wave; m <<= 1) {
 #pragma unroll
@@ -395,7 +434,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
 #pragma unroll
                         for (int v = 0; v < VEC; v++) acc[v] = fmaxf(acc[v], 0.0f);
                     }
-                    store_vec<VEC>(Y + out_row * ld + col, acc);
+                    store_vec_streaming<VEC>(Y + out_row * ld + col, acc, N * 4 >= ACCEL_STREAMING_MIN_BYTES);
                 }
             }
         }
@@ -467,7 +506,7 @@ __global__ __launch_bounds__(256) void copy_u32_kernel(uint32_t *__restrict__ ds
         dst[i] = src[i];
 }
 
-template <int VEC>
+template <int VEC, bool kWide>
 int launch_for_vec(bool team, int L, dim3 grid, hipStream_t s, const int4 *work, int n_units,
                    const int32_t *s_idx, const float *s_val, const int32_t *perm, const float *X,
                    float *Y, float *partial, int N, int ld, int n_zero_rows, int n_zero_groups,
@@ -476,11 +515,11 @@ int launch_for_vec(bool team, int L, dim3 grid, hipStream_t s, const int4 *work,
 #define ACCEL_LAUNCH(LL)                                                                      \
     case LL:                                                                                  \
         if (team)                                                                             \
-            spmm_team_kernel<LL, VEC><<<grid, dim3(kWgThreads), 0, s>>>(                      \
+            spmm_team_kernel<LL, VEC, kWide><<<grid, dim3(kWgThreads), 0, s>>>(                      \
                 work, n_units, s_idx, s_val, perm, X, Y, partial, N, ld, n_zero_rows,         \
                 n_zero_groups, bias, relu);                                                   \
         else                                                                                  \
-            spmm_gather_kernel<LL, VEC><<<grid, dim3(kWgThreads), 0, s>>>(                    \
+            spmm_gather_kernel<LL, VEC, kWide><<<grid, dim3(kWgThreads), 0, s>>>(                    \
                 work, n_units, s_idx, s_val, perm, X, Y, partial, N, ld, n_zero_rows,         \
                 n_zero_groups, bias, relu);                                                   \
         break;
@@ -557,6 +596,8 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     if (kPanel > 0 && vec == 4 && N > kPanel && N % kPanel == 0 && h->nnz >= kPanelMinNnz &&
         h->nnz >= 16 * h->rows)
         panel = kPanel;
+    // operands below 4 GiB are addressed with 32-bit byte offsets (see gather_row)
+    const bool wide = (uint64_t)h->cols * (uint64_t)N * 4u > 0xFFFFFFFFull;
     const int4 *wk = reinterpret_cast<const int4 *>(h->work);
     const int64_t entry_groups = h->plan_team ? h->n_units : h->n_units / kWaves;
     for (int c0 = 0; c0 < N; c0 += panel) {
@@ -579,15 +620,17 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         float *Yp = Y + c0, *Pp = h->partial ? h->partial + c0 : nullptr;
         const float *bp = bias ? bias + c0 : nullptr;
         int rc;
-        if (vec == 4)
-            rc = launch_for_vec<4>(h->plan_team, L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
-                                   Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu);
-        else if (vec == 2)
-            rc = launch_for_vec<2>(h->plan_team, L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
-                                   Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu);
-        else
-            rc = launch_for_vec<1>(h->plan_team, L, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm, Xp,
-                                   Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu);
+#define ACCEL_DISPATCH(V)                                                                              \
+    (wide ? launch_for_vec<V, true>(h->plan_team, L, grid, stream, wk, (int)h->n_units, h->s_idx,       \
+                                    h->s_val, h->perm, Xp, Yp, Pp, n, N, (int)h->n_zero_rows,          \
+                                    (int)zero_groups, bp, relu)                                        \
+          : launch_for_vec<V, false>(h->plan_team, L, grid, stream, wk, (int)h->n_units, h->s_idx,      \
+                                     h->s_val, h->perm, Xp, Yp, Pp, n, N, (int)h->n_zero_rows,         \
+                                     (int)zero_groups, bp, relu))
+        if (vec == 4) rc = ACCEL_DISPATCH(4);
+        else if (vec == 2) rc = ACCEL_DISPATCH(2);
+        else rc = ACCEL_DISPATCH(1);
+#undef ACCEL_DISPATCH
         if (rc) return rc;
     }
     if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));
