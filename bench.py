@@ -180,6 +180,13 @@ def main():
     ap.add_argument("--compare-neighbor-partition", action="store_true",
                     help="also time a neighbour-partition kernel with atomics (the scheme of "
                          "upstream's spmm_gnna.cu) on the same operands (comparison only)")
+    ap.add_argument("--gather-probe", type=int, default=0, metavar="ROWS",
+                    help="only run the pure-gather probe: random rows of --N floats (16, 64 or 256) "
+                         "from an array of ROWS rows, with --probe-stores none|plain|streaming and one "
+                         "stored row per --probe-row-len gathers (what the GPU sustains for the SpMM's "
+                         "access pattern when a kernel does nothing else)")
+    ap.add_argument("--probe-stores", default="none", choices=["none", "plain", "streaming"])
+    ap.add_argument("--probe-row-len", type=int, default=32)
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run the plain copy kernel over this many MiB, --steps times "
                          "(known-size reference for the FETCH_SIZE / WRITE_SIZE counters)")
@@ -192,6 +199,24 @@ def main():
     pkg = entry.load_package()
     if pkg.device_count() < 1:
         sys.exit("bench.py: no GPU: " + pkg._lib.last_error())
+    if a.gather_probe:
+        import ctypes as C
+        L = C.CDLL(os.path.join(os.path.dirname(str(pkg._lib.LIB_PATH)), "libaccelgcn_baselines.so"))
+        L.baseline_gather_probe_last_error.restype = C.c_char_p
+        N = a.N or 64
+        ms, gathered, stored = C.c_float(0), C.c_double(0), C.c_double(0)
+        stores = {"none": 0, "plain": 1, "streaming": 2}[a.probe_stores]
+        rc = L.baseline_gather_probe(C.c_int64(a.gather_probe), C.c_int32(N), C.c_int32(256),
+                                     C.c_int32(a.probe_row_len), C.c_int32(stores), C.c_int32(5),
+                                     C.byref(ms), C.byref(gathered), C.byref(stored))
+        if rc != 0:
+            sys.exit("bench.py: gather probe: " + L.baseline_gather_probe_last_error().decode())
+        print(json.dumps({"gather_probe": {"rows_of_X": a.gather_probe, "N": N, "X_MB": round(a.gather_probe * N * 4 / 1e6, 2),
+                                            "stores": a.probe_stores, "gathers_per_stored_row": a.probe_row_len,
+                                            "ms": round(ms.value, 4),
+                                            "gathered_TB_per_s": round(gathered.value / ms.value / 1e9, 2),
+                                            "stored_TB_per_s": round(stored.value / ms.value / 1e9, 3)}}), flush=True)
+        return
     if a.copy_calibration:
         import ctypes as C
         words = a.copy_calibration * (1 << 20) // 4

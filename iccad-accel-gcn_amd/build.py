@@ -73,11 +73,12 @@ def build(verbose: bool = False, extra_flags=(), out: Path | None = None) -> Pat
 
 def build_baselines(verbose: bool = False) -> Path:
     """lib/libaccelgcn_baselines.so: comparison baselines (rocSPARSE SpMM and a
-    neighbour-partition kernel).  Kept in its own library: the product library does
+    neighbour-partition kernel) and the pure-gather measurement probe.  Kept in its own library: the product library does
     not link any sparse library and holds no comparison code."""
     out = LIB_DIR / "libaccelgcn_baselines.so"
     cmd = [hipcc(), *compile_flags(), "-shared", str(PKG / "baselines" / "rocsparse_spmm.cpp"),
-           str(PKG / "baselines" / "neighbor_partition_spmm.cpp"), "-o", str(out), "-lrocsparse"]
+           str(PKG / "baselines" / "neighbor_partition_spmm.cpp"),
+           str(PKG / "baselines" / "gather_probe.cpp"), "-o", str(out), "-lrocsparse"]
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

@@ -64,3 +64,18 @@ def test_rocsparse_baseline_computes_the_product(gpu, baselines):
     assert so.check(Y, g.indptr, g.indices, g.values, X) <= so.TOL
     for b in bufs + [dY]:
         b.close()
+
+
+def test_gather_probe_runs(gpu, baselines):
+    """The pure-gather measurement probe: argument checks and a small run."""
+    baselines.baseline_gather_probe_last_error.restype = C.c_char_p
+    ms, gathered, stored = C.c_float(0), C.c_double(0), C.c_double(0)
+    for stores in (0, 1, 2):
+        rc = baselines.baseline_gather_probe(C.c_int64(1000), C.c_int32(64), C.c_int32(8), C.c_int32(4),
+                                             C.c_int32(stores), C.c_int32(1), C.byref(ms), C.byref(gathered),
+                                             C.byref(stored))
+        assert rc == 0, baselines.baseline_gather_probe_last_error().decode()
+        assert ms.value > 0 and gathered.value == 65536 * 4 * 8 * 256.0
+        assert (stored.value > 0) == (stores != 0)
+    assert baselines.baseline_gather_probe(C.c_int64(1000), C.c_int32(48), C.c_int32(8), C.c_int32(4), C.c_int32(0),
+                                           C.c_int32(1), C.byref(ms), None, None) != 0      # N must be 16, 64 or 256
