@@ -108,6 +108,7 @@ struct accel_handle {
     int plan_groups = 0;              // 0: by row length (row_groups); 8..64: the same for all rows
     int plan_team_option = 0;         // 0: choose from the size of the matrix; 1: wavefront units; 2: workgroup units
     bool plan_team = false;           // a unit is worked on by a whole workgroup (small matrices)
+    bool local = false;               // most non-zeros lie near the diagonal (sampled)
     int64_t n_split_rows = 0;         // rows with more than plan_split non-zeros
     int64_t n_big_rows = 0;           // of those, rows with more than 32 * plan_split
     int64_t n_blocks = 0, n_long_blocks = 0, n_long_rows = 0, n_zero_rows = 0;

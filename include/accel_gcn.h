@@ -115,7 +115,8 @@ int accel_preprocess(accel_handle *h);
  * never changes.  Call before accel_preprocess. */
 int accel_set_plan_unit(accel_handle *h, int unit_nz);
 /* Rows with more non-zeros than this (16..384, never above the unit size; 0 = let
- * the library choose) are the ones stored by column group and cut into pieces. */
+ * the library choose: 192, or 384 when most non-zeros of the matrix lie near its
+ * diagonal) are the ones stored by column group and cut into pieces. */
 int accel_set_plan_split(accel_handle *h, int split_nz);
 /* Number of column groups the pieces of split rows are sorted into: 8, 16, 32 or
  * 64 for every row, or 0 (the default) to choose per row: 8 groups, doubled while

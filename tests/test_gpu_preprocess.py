@@ -312,6 +312,35 @@ def test_launch_plan_row_bands(gpu):
     op.close()
 
 
+def test_near_diagonal_matrices_keep_mid_rows_whole(gpu):
+    """The split threshold is 192 for a large matrix, unless most of its non-zeros lie near the
+    diagonal: then rows of up to 384 non-zeros stay whole (sampled on the GPU)."""
+    from oracle import spmm_oracle as so
+    rng = np.random.default_rng(33)
+    n, d = 60_000, 10
+    deg = np.full(n, d)
+    deg[rng.integers(0, n, 300)] = rng.integers(200, 380, 300)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    rows_of = np.repeat(np.arange(n), deg)
+    values = rng.uniform(-1, 1, rows_of.size).astype(np.float32)
+    X = rng.uniform(-1, 1, (n, 16)).astype(np.float32)
+    for kind, want in (("band", 384), ("uniform", 192)):
+        if kind == "band":
+            cols = np.clip(rows_of + rng.integers(-600, 601, rows_of.size), 0, n - 1)
+        else:
+            cols = rng.integers(0, n, rows_of.size)
+        op = gpu.AccelSpMM(indptr, cols.astype(np.int32), values, n).preprocess()
+        assert op.info.nnz >= 512 * 1024 and op.info.plan_team == 0
+        assert op.info.plan_split_nz == want, kind
+        assert op.info.n_split_rows == int((deg > want).sum())
+        assert so.check(op.matmul(X), indptr, cols.astype(np.int32), values, X) <= so.TOL
+        op.close()
+    # an explicit threshold is never overridden
+    op = gpu.AccelSpMM(indptr, cols.astype(np.int32), values, n).preprocess(plan_split=100)
+    assert op.info.plan_split_nz == 100
+    op.close()
+
+
 def test_launch_plan_hub_graph(gpu):
     g = gpu.synthetic.hub_graph_small()
     op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
