@@ -290,14 +290,17 @@ def test_fused_bias_and_relu(gpu, mixed, N):
         buf.close()
 
 
-def test_operands_beyond_4_gib(gpu):
-    """X and Y larger than 4 GiB: row offsets need 64-bit arithmetic.  The
-    matrix references rows of X at both ends of a 5.1 GB buffer and writes rows
+@pytest.mark.parametrize("n_cols,team", [(5_000_000, 2), (5_000_000, 1), (4_194_300, 1)])
+def test_operands_beyond_4_gib(gpu, n_cols, team):
+    """X and Y larger than 4 GiB: row offsets need 64-bit arithmetic (both kernels), and an X
+    just below 4 GiB, the largest that is addressed with 32-bit byte offsets.  The
+    matrix references rows of X at both ends of a 5.1 (4.3) GB buffer and writes rows
     of Y at both ends of a 4.4 GB buffer; only the touched rows travel to the host."""
     import ctypes as C
-    N, n_cols, n_rows = 256, 5_000_000, 4_300_000
+    N, n_rows = 256, 4_300_000
+    assert (n_cols * N * 4 > 2 ** 32) == (n_cols == 5_000_000)
     rng = np.random.default_rng(0)
-    cols = np.unique(np.concatenate([[0, 1, n_cols - 1, n_cols - 2, 4_194_304, 4_194_303],
+    cols = np.unique(np.concatenate([[0, 1, n_cols - 1, n_cols - 2, min(4_194_304, n_cols - 3), 4_194_203],
                                      rng.integers(0, n_cols, 500)])).astype(np.int32)
     live_rows = np.unique(np.concatenate([[0, 7, n_rows - 1, n_rows - 2, 4_194_304, 4_194_305],
                                           rng.integers(0, n_rows, 60)]))
@@ -318,7 +321,7 @@ def test_operands_beyond_4_gib(gpu):
     dY.fill_u32(0x7FC00000)
     for c, row in zip(cols, Xrows):                            # only the referenced rows of X are non-zero
         gpu._lib.check(lib.accel_memcpy_h2d(C.c_void_p(dX.address + int(c) * N * 4), C.c_void_p(row.ctypes.data), N * 4))
-    op = gpu.AccelSpMM(indptr.astype(np.int32), idx, val, n_cols).preprocess()
+    op = gpu.AccelSpMM(indptr.astype(np.int32), idx, val, n_cols).preprocess(plan_team=team)
     op.run(dX, dY, N)
     op.synchronize()
 
