@@ -1,4 +1,4 @@
-// The SpMM gather kernel for gfx950 (wave64) and its two helpers.
+// The SpMM gather kernels for gfx950 (wave64), the partial-sum reduction and two helpers.
 //
 // Work decomposition.  Upstream gives one CUDA thread block of 12 32-lane warps
 // to each block4 entry (spmm_accel.cu:18-28).  Here one 64-lane wavefront takes
@@ -7,9 +7,10 @@
 // total) or a piece of <= 384 non-zeros of a split row (every row with more than
 // 384 non-zeros is split; the plan also splits somewhat shorter ones).  The units
 // come from a launch plan built by the preprocessing step; it orders them so that
-// workgroup i, which the hardware places on die i % 8, works on a column group
-// (share of X) that die keeps in its own L2.  Small matrices use the same list with
-// one unit per workgroup instead (spmm_team_kernel below).
+// workgroup i, which the hardware places on die i % 8, works on a share of X that
+// die keeps in its own L2: a column group for the pieces of split rows, a band of
+// the caller's rows for the whole-row units.  Small matrices use the same list
+// with one unit per workgroup instead (spmm_team_kernel below).
 //
 // Inside the wavefront the lanes form G = 64 / L groups of L lanes; a group owns
 // L * VEC consecutive columns of X/Y (VEC = 4 floats = one 16-byte load per lane
