@@ -226,7 +226,7 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
 }
 
 // Does the matrix have its non-zeros near the diagonal (of the rows x cols rectangle)?
-// Every kLocalityStride-th row contributes up to kLocalitySample of its non-zeros; one counts
+// Every kLocalityStride-th row contributes up to kLocalitySample of its non-zeros, evenly spaced; one counts
 // as local when its column is within `band` columns of the row's place.  Runs after indptr
 // has been validated.
 constexpr int kLocalityStride = 16, kLocalitySample = 16;
@@ -237,10 +237,10 @@ __global__ __launch_bounds__(kThreads) void locality_kernel(const int32_t *__res
     const int64_t r = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * kLocalityStride;
     int seen = 0, local = 0;
     if (r < rows) {
-        const int a = indptr[r], n = min(indptr[r + 1] - a, kLocalitySample);
+        const int a = indptr[r], d = indptr[r + 1] - a, n = min(d, kLocalitySample);
         const int64_t place = rows > 1 ? r * (cols - 1) / (rows - 1) : 0;
-        for (int i = 0; i < n; i++) {
-            const int64_t off = (int64_t)idx[a + i] - place;
+        for (int i = 0; i < n; i++) {                    // spread over the row, whatever its order
+            const int64_t off = (int64_t)idx[a + (int)((int64_t)i * d / n)] - place;
             local += (off < 0 ? -off : off) <= band;
         }
         seen = n;
