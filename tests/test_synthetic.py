@@ -55,3 +55,42 @@ def test_dense_operand(pkg):
     assert np.array_equal(X, pkg.synthetic.dense_operand("cfg2", 100, 16))
     Z = pkg.synthetic.dense_operand("cfg5", 2000, 8)
     assert abs(Z.mean()) < 0.05 and abs(Z.std() - 1) < 0.05
+
+
+def _bench_module():
+    import importlib.util
+    import os
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py")
+    spec = importlib.util.spec_from_file_location("bench_under_test", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_bench_fixture_graphs_keep_the_golden_degree_sequence(pkg):
+    """bench.py's fixture:<g> and local:<g>:<sigma> workloads: the degree sequence is the one
+    the golden .block4 file of <g> encodes; local columns stay near the row id."""
+    import sys, os
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    import block4_codec
+    from oracle import partition_oracle as po
+    bench = _bench_module()
+    golden = block4_codec.load("pubmed")
+    want = np.sort(po.degrees_from_block4(golden))
+    g = bench.fixture_graph(pkg, "pubmed")
+    well_formed(g)
+    # duplicates inside a row merge, so a row may fall slightly short of its target degree
+    got = np.sort(np.diff(g.indptr))
+    assert got.size == want.size and np.all(got <= want) and got.sum() >= 0.999 * want.sum()
+    loc = bench.fixture_graph(pkg, "pubmed", sigma=50)
+    well_formed(loc)
+    rows = np.repeat(np.arange(loc.n_rows), np.diff(loc.indptr))
+    assert np.percentile(np.abs(loc.indices - rows), 99) <= 3 * 50 + 1
+    assert np.abs(g.indices - np.repeat(np.arange(g.n_rows), np.diff(g.indptr))).mean() > 1000
+
+
+def test_bench_uniform_probe_graph(pkg):
+    bench = _bench_module()
+    g = bench.uniform_graph(pkg, 1000, 7, 300)
+    assert g.n_rows == 1000 and g.n_cols == 300 and g.nnz == 7000
+    assert np.all(np.diff(g.indptr) == 7) and g.indices.min() >= 0 and g.indices.max() < 300
