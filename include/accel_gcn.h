@@ -124,7 +124,8 @@ int accel_set_plan_split(accel_handle *h, int split_nz);
  * (column >> 3) & (groups - 1) is worked on by die g % 8, one group after the
  * other.  Call before accel_preprocess. */
 int accel_set_plan_groups(accel_handle *h, int groups);
-/* Who works on one unit of the launch plan: 1 = one wavefront (four units per
+/* Who works on one unit of the launch plan (no counterpart upstream, where a block4
+ * entry always gets one thread block, spmm_accel.cu:128): 1 = one wavefront (four units per
  * workgroup, the layout described at accel_get_plan); 2 = a whole workgroup of four
  * wavefronts, which share the unit's rows or, for a long row, its non-zeros; 0 (the
  * default) = the library chooses: workgroup units for small matrices, whose run time
