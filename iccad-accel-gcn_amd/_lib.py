@@ -21,6 +21,7 @@ PTR_HOST, PTR_DEVICE = 0, 1
 EPILOGUE_RELU = 1
 DEG_BOUND = 384
 SLICES_PER_BLOCK = 12
+STATIC_SCRATCH_BYTES = 32 << 20
 
 _STATUS_NAME = {ERR_ARG: "ACCEL_ERR_ARG", ERR_CSR: "ACCEL_ERR_CSR", ERR_ALLOC: "ACCEL_ERR_ALLOC",
                 ERR_HIP: "ACCEL_ERR_HIP", ERR_META: "ACCEL_ERR_META", ERR_STATE: "ACCEL_ERR_STATE",
@@ -79,6 +80,7 @@ SIGNATURES = {
     "accel_get_perm": (C.c_int, [vp, i32p, C.c_int64]),
     "accel_get_sorted_csr": (C.c_int, [vp, i32p, i32p, f32p]),
     "accel_run": (C.c_int, [vp, vp, vp, C.c_int32, vp]),
+    "accel_run_static": (C.c_int, [vp, vp, vp, C.c_int32, vp]),
     "accel_run_epilogue": (C.c_int, [vp, vp, vp, C.c_int32, vp, C.c_int, vp]),
     "accel_time": (C.c_int, [vp, vp, vp, C.c_int32, C.c_int, C.c_int, f32p, f32p, vp]),
     "accel_destroy": (C.c_int, [vp]),

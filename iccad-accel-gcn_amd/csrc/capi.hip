@@ -561,6 +561,16 @@ int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream
     return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr);
 }
 
+int accel_run_static(accel_handle *h, const float *X, float *Y, int32_t N, void *stream)
+{
+    clear_error();
+    if (!h) { set_error("accel_run_static: null handle"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_run_static: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (N <= 0) { set_error("accel_run_static: N must be positive, got %d", N); return ACCEL_ERR_ARG; }
+    if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("accel_run_static: null dense operand"); return ACCEL_ERR_ARG; }
+    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, nullptr, 0, true);
+}
+
 int accel_run_epilogue(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias,
                        int flags, void *stream)
 {

@@ -124,7 +124,8 @@ namespace accel {
 int preprocess_device(accel_handle *h);
 // spmm.hip
 int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
-                hipEvent_t after_main, const float *bias = nullptr, int relu = 0);
+                hipEvent_t after_main, const float *bias = nullptr, int relu = 0,
+                bool static_partial = false);
 int fill_u32(void *dst, uint32_t v, size_t n, hipStream_t s);
 int copy_u32(void *dst, const void *src, size_t n, hipStream_t s);
 }  // namespace accel

@@ -28,7 +28,18 @@
 // scratch buffer and a second small kernel adds them up in a fixed order, so the
 // result is run-to-run deterministic.  Rows of degree 0 are zero-filled by extra
 // workgroups of the same launch: Y = A X holds after every run with no memset.
+#include <mutex>
+
 #include "internal.h"
+
+// Partial sums for accel_run_static, the entry point that allocates nothing: one copy of
+// this array per GPU, held from the moment the library's code is loaded on that GPU until
+// the process ends.  In host code the name is only a handle for the runtime, not a device
+// address: static_scratch_address() asks for the address once per GPU and everything else
+// (kernel arguments included) uses that pointer.
+static constexpr size_t kStaticScratchFloats = (size_t)ACCEL_STATIC_SCRATCH_BYTES / sizeof(float);
+static constexpr int kMaxScratchDevices = 64;
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
 
 namespace accel {
 namespace {
@@ -562,8 +573,31 @@ int copy_u32(void *dst, const void *src, size_t n, hipStream_t s)
     return ACCEL_OK;
 }
 
+// Device address of this GPU's copy of `scratch`, looked up once per device (with that
+// device current) and kept.
+static int static_scratch_address(float **out)
+{
+    static std::mutex mu;
+    static float *addr[kMaxScratchDevices] = {};
+    int dev = 0;
+    ACCEL_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxScratchDevices) {
+        set_error("device ordinal %d is beyond the %d devices the static scratch is tracked for", dev,
+                  kMaxScratchDevices);
+        return ACCEL_ERR_ARG;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!addr[dev]) {
+        float *p = nullptr;
+        ACCEL_HIP(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
+        addr[dev] = p;
+    }
+    *out = addr[dev];
+    return ACCEL_OK;
+}
+
 int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
-                hipEvent_t after_main, const float *bias, int relu)
+                hipEvent_t after_main, const float *bias, int relu, bool static_partial)
 {
     if (h->rows == 0) return ACCEL_OK;
     // widest vector the row stride and the base pointers allow
@@ -572,7 +606,21 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     if (N % 4 == 0 && align % 16 == 0) vec = 4;
     else if (N % 2 == 0 && align % 8 == 0) vec = 2;
 
-    if (h->n_long_units > 0) {
+    // partial sums of the pieces of split rows: the handle's buffer (allocated here when a
+    // run needs more than it holds), or this GPU's static array, which is never allocated
+    float *partial = h->partial;
+    if (static_partial) {
+        partial = nullptr;
+        const size_t need = (size_t)h->n_long_units * (size_t)N;
+        if (need > kStaticScratchFloats) {
+            set_error("accel_run_static: this matrix needs %zu floats of partial sums at N = %d "
+                      "(%lld pieces of split rows x N), the static scratch holds %zu",
+                      need, N, (long long)h->n_long_units, kStaticScratchFloats);
+            return ACCEL_ERR_ARG;
+        }
+        if (need > 0)
+            if (int rc = static_scratch_address(&partial)) return rc;
+    } else if (h->n_long_units > 0) {
         const size_t need = (size_t)h->n_long_units * (size_t)N;
         if (h->partial_floats < need) {
             if (h->partial) (void)hipFree(h->partial);
@@ -586,6 +634,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
             }
             h->partial_floats = need;
         }
+        partial = h->partial;
     }
     // Wide operands are computed one column panel at a time (all units for the first
     // panel, then all units for the next): a panel's slice of X is what the L2s have
@@ -619,7 +668,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         if (groups == 0) break;
         const dim3 grid((unsigned)groups);
         const float *Xp = X ? X + c0 : X;
-        float *Yp = Y + c0, *Pp = h->partial ? h->partial + c0 : nullptr;
+        float *Yp = Y + c0, *Pp = partial ? partial + c0 : nullptr;
         const float *bp = bias ? bias + c0 : nullptr;
         int rc;
 #define ACCEL_DISPATCH(V)                                                                              \
@@ -643,7 +692,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         const int rpw = N <= 64 ? 4 : N <= 128 ? 2 : 1;
         const int shared_groups = (n_shared + rpw - 1) / rpw;
         long_row_reduce_kernel<<<dim3((unsigned)(shared_groups + n_big)), dim3(kReduceThreads), 0, stream>>>(
-            h->partial, h->long_slot, h->perm, h->rows - h->n_split_rows, n_shared, shared_groups, rpw,
+            partial, h->long_slot, h->perm, h->rows - h->n_split_rows, n_shared, shared_groups, rpw,
             n_split, Y, N, bias, relu);
     }
     ACCEL_HIP(hipGetLastError());

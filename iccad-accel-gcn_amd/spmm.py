@@ -126,6 +126,12 @@ class AccelSpMM:
         """One asynchronous launch; X, Y are device buffers."""
         check(lib().accel_run(self._h, ptr(X), ptr(Y), int(N), ptr(stream)))
 
+    def run_static(self, X, Y, N: int, stream=None) -> None:
+        """``run`` without any device allocation: the partial sums of split rows go to
+        the library's static scratch array (ACCEL_STATIC_SCRATCH_BYTES per GPU) and a
+        matrix that needs more at this N is refused (see accel_run_static)."""
+        check(lib().accel_run_static(self._h, ptr(X), ptr(Y), int(N), ptr(stream)))
+
     def run_epilogue(self, X, Y, N: int, bias=None, relu=False, stream=None) -> None:
         """Y = act(A X + bias) in one launch; bias is a device buffer of N floats or None."""
         check(lib().accel_run_epilogue(self._h, ptr(X), ptr(Y), int(N), ptr(bias),

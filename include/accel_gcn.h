@@ -197,6 +197,22 @@ int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream
 int accel_run_epilogue(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias,
                        int flags, void *stream);
 
+/* accel_run for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart upstream.  The only scratch of a run, the partial sums of the
+ * pieces of split rows (pieces x N floats), lives in a static device array of
+ * ACCEL_STATIC_SCRATCH_BYTES that every GPU the library runs on holds until the
+ * process ends, instead of the handle's buffer that accel_run allocates on its
+ * first call with a given N.  This call allocates and frees nothing.  A matrix
+ * whose partial sums at this N do not fit is refused with ACCEL_ERR_ARG and a
+ * message that names both sizes (matrices without split rows need none and always
+ * fit).  All handles on one GPU share the array: two calls that overlap in time
+ * on the same GPU (different streams or different handles) race; calls queued on
+ * one stream are safe.  Every slot a run reads is written by that run first, so
+ * nothing needs clearing between calls.  Same result, bit for bit, as accel_run. */
+#define ACCEL_STATIC_SCRATCH_BYTES (32u << 20)
+int accel_run_static(accel_handle *h, const float *X, float *Y, int32_t N, void *stream);
+
 /* Timing protocol of SPMM_BASE::timing_body (spmm_base.h:34-63) with HIP
  * events on `stream`: `warmup` untimed runs, then `iters` runs each bracketed
  * by events.  ms_total[i] covers everything accel_run launches; ms_main[i]
