@@ -7,14 +7,12 @@ CPU stand-in for any GPU entry point.
 from __future__ import annotations
 
 import ctypes as C
-import os
 from pathlib import Path
 
 import numpy as np
 
 PKG = Path(__file__).resolve().parent
-# ACCEL_GCN_LIB selects another build of the same library (e.g. a tuning variant)
-LIB_PATH = Path(os.environ.get("ACCEL_GCN_LIB") or PKG / "lib" / "libaccelgcn.so")
+LIB_PATH = PKG / "lib" / "libaccelgcn.so"
 
 OK, ERR_ARG, ERR_CSR, ERR_ALLOC, ERR_HIP, ERR_META, ERR_STATE, ERR_IO = 0, -1, -2, -3, -4, -5, -6, -7
 PTR_HOST, PTR_DEVICE = 0, 1
@@ -73,6 +71,7 @@ SIGNATURES = {
     "accel_set_plan_groups": (C.c_int, [vp, C.c_int]),
     "accel_set_plan_split": (C.c_int, [vp, C.c_int]),
     "accel_set_plan_team": (C.c_int, [vp, C.c_int]),
+    "accel_set_plan_panel": (C.c_int, [vp, C.c_int]),
     "accel_check_block4": (C.c_int, [vp, i32p, C.c_int64]),
     "accel_get_info": (C.c_int, [vp, C.POINTER(Info)]),
     "accel_get_block4": (C.c_int, [vp, i32p, C.c_int64]),

@@ -394,6 +394,19 @@ int accel_set_plan_team(accel_handle *h, int mode)
     return ACCEL_OK;
 }
 
+int accel_set_plan_panel(accel_handle *h, int columns)
+{
+    clear_error();
+    if (!h) { set_error("accel_set_plan_panel: null handle"); return ACCEL_ERR_ARG; }
+    if (columns != 0 && (columns < 4 || columns > 1024 || columns % 4 != 0)) {
+        set_error("accel_set_plan_panel: width must be 0 (automatic) or a multiple of 4 in 4..1024, got %d",
+                  columns);
+        return ACCEL_ERR_ARG;
+    }
+    h->plan_panel_option = columns;
+    return ACCEL_OK;
+}
+
 int accel_preprocess(accel_handle *h)
 {
     clear_error();

@@ -107,6 +107,7 @@ struct accel_handle {
     int plan_split = ACCEL_DEG_BOUND; // rows with more non-zeros than this are cut into pieces (<= plan_unit)
     int plan_groups = 0;              // 0: by row length (row_groups); 8..64: the same for all rows
     int plan_team_option = 0;         // 0: choose from the size of the matrix; 1: wavefront units; 2: workgroup units
+    int plan_panel_option = 0;        // 0: choose; else the column-panel width of wide operands
     bool plan_team = false;           // a unit is worked on by a whole workgroup (small matrices)
     bool local = false;               // most non-zeros lie near the diagonal (sampled)
     int64_t n_split_rows = 0;         // rows with more than plan_split non-zeros

@@ -53,81 +53,54 @@ constexpr int kReduceThreads = 256;       // workgroup of the partial-sum reduct
 // a workgroup's share is a whole number of vectors)
 __host__ __device__ inline int zero_rows_per_group(int N) { return N >= kZeroFloats ? 1 : kZeroFloats / N; }
 
-// build-time tuning knobs (defaults are the measured best)
-#ifndef ACCEL_UNROLL
-#define ACCEL_UNROLL 4                    // gathers in flight per lane in the main loop
-#endif
-#ifndef ACCEL_PANEL
-#define ACCEL_PANEL 64                    // column-panel width for wide operands (0: never split)
-#endif
-#ifndef ACCEL_PANEL_MIN_NNZ
-#define ACCEL_PANEL_MIN_NNZ 4000000       // smaller matrices are not worth several launches
-#endif
-#ifndef ACCEL_TEAM_UNROLL
-#define ACCEL_TEAM_UNROLL 4               // the same for the kernel with workgroup units (8: 5-10 % slower)
-#endif
-#ifndef ACCEL_STREAMING_STORES
-#define ACCEL_STREAMING_STORES 1
-#endif
-#ifndef ACCEL_STREAMING_MIN_BYTES
-#define ACCEL_STREAMING_MIN_BYTES 64         // rows of Y of at least this many bytes are stored streaming
-                                             // (64-byte rows: L2-resident X -18 %, elsewhere within 1 %)
-#endif
-constexpr int kUnroll = ACCEL_UNROLL;
-constexpr int kTeamUnroll = ACCEL_TEAM_UNROLL;
-constexpr int kPanel = ACCEL_PANEL;
-constexpr int64_t kPanelMinNnz = ACCEL_PANEL_MIN_NNZ;
+constexpr int kUnroll = 4;                // gathers in flight per lane in the main loop (2 and 8 measured within 2 %)
+constexpr int kTeamUnroll = 4;            // the same with workgroup units (8: 5-10 % slower)
+constexpr int kPanel = 64;                // column-panel width for wide operands on large matrices
+constexpr int kPanelMinNnz = 4000000;     // smaller matrices are not worth several launches
+constexpr int kStreamingMinBytes = 64;    // rows of Y of at least this many bytes are stored streaming
+                                          // (64-byte rows: L2-resident X -18 %, elsewhere within 1 %)
 
-template <int VEC>
+// A vector of four floats that is only 4-byte aligned: rows of X and Y start at any
+// multiple of 4 bytes when N is not a multiple of 4.  The hardware takes 16-byte
+// accesses at such addresses; the type keeps the compiler from assuming more.
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef v4f v4f_unaligned __attribute__((aligned(4)));
+
+template <int VEC, bool kShift>
 __device__ __forceinline__ void load_vec(const float *__restrict__ p, float (&v)[VEC])
 {
-    if constexpr (VEC == 4) {
+    if constexpr (VEC == 4 && kShift) {
+        const v4f t = *reinterpret_cast<const v4f_unaligned *>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else if constexpr (VEC == 4) {
         const float4 t = *reinterpret_cast<const float4 *>(p);
         v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-    } else if constexpr (VEC == 2) {
-        const float2 t = *reinterpret_cast<const float2 *>(p);
-        v[0] = t.x; v[1] = t.y;
     } else {
+        static_assert(VEC == 1, "vector widths: 4 or 1");
         v[0] = *p;
     }
 }
 
-template <int VEC>
-__device__ __forceinline__ void store_vec(float *__restrict__ p, const float (&v)[VEC])
+// Rows of Y are written once and not read again by this launch: a streaming
+// (non-temporal) store when `streaming`.  Measured on this GPU with gathers that hit L2:
+// one ordinary 256-byte store per 32 gathers lowers the gather rate from 27 to 20 TB/s, a
+// non-temporal one to 26 TB/s.
+template <int VEC, bool kShift>
+__device__ __forceinline__ void store_vec(float *__restrict__ p, const float (&v)[VEC], bool streaming)
 {
     if constexpr (VEC == 4) {
-        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
-    } else if constexpr (VEC == 2) {
-        *reinterpret_cast<float2 *>(p) = make_float2(v[0], v[1]);
-    } else {
-        *p = v[0];
-    }
-}
-
-// Rows of Y are written once and not read again by this launch: a streaming
-// (non-temporal) store.  Measured on this GPU with gathers that hit L2: one ordinary
-// 256-byte store per 32 gathers lowers the gather rate from 27 to 20 TB/s, a
-// non-temporal one to 26 TB/s.
-template <int VEC>
-__device__ __forceinline__ void store_vec_streaming(float *__restrict__ p, const float (&v)[VEC], bool streaming)
-{
-#if ACCEL_STREAMING_STORES
-    if (!streaming) {
-        store_vec<VEC>(p, v);
-    } else if constexpr (VEC == 4) {
-        typedef float v4f __attribute__((ext_vector_type(4)));
         const v4f t = {v[0], v[1], v[2], v[3]};
-        __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
-    } else if constexpr (VEC == 2) {
-        typedef float v2f __attribute__((ext_vector_type(2)));
-        const v2f t = {v[0], v[1]};
-        __builtin_nontemporal_store(t, reinterpret_cast<v2f *>(p));
+        if constexpr (kShift) {
+            if (streaming) __builtin_nontemporal_store(t, reinterpret_cast<v4f_unaligned *>(p));
+            else *reinterpret_cast<v4f_unaligned *>(p) = t;
+        } else {
+            if (streaming) __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
+            else *reinterpret_cast<v4f *>(p) = t;
+        }
     } else {
-        __builtin_nontemporal_store(v[0], p);
+        if (streaming) __builtin_nontemporal_store(v[0], p);
+        else *p = v[0];
     }
-#else
-    store_vec<VEC>(p, v);
-#endif
 }
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
@@ -138,7 +111,7 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 // The staged pair holds the value and, when the operand is smaller than 4 GiB (kWide ==
 // false), the byte offset of the row of X, so that the address is one 32-bit add to a
 // uniform base; otherwise the column, and the address is formed with 64-bit arithmetic.
-template <int VEC, int U, bool kWide>
+template <int VEC, int U, bool kWide, bool kShift>
 __device__ __forceinline__ void gather_row(const int2 *__restrict__ row_st, int d, int k, int gp,
                                            const float *__restrict__ X, int col, int ld,
                                            float (&acc)[VEC])
@@ -147,9 +120,9 @@ __device__ __forceinline__ void gather_row(const int2 *__restrict__ row_st, int 
     const uint32_t lane_off = (uint32_t)col * 4u;
     auto fetch = [&](int where, float (&x)[VEC]) {
         if constexpr (kWide)
-            load_vec<VEC>(X + col + (int64_t)where * ld, x);
+            load_vec<VEC, kShift>(X + col + (int64_t)where * ld, x);
         else
-            load_vec<VEC>(reinterpret_cast<const float *>(xb + ((uint32_t)where + lane_off)), x);
+            load_vec<VEC, kShift>(reinterpret_cast<const float *>(xb + ((uint32_t)where + lane_off)), x);
     };
     int o = k;
     for (; o + (U - 1) * gp < d; o += U * gp) {          // full batches
@@ -211,11 +184,11 @@ __device__ __forceinline__ void zero_fill_rows(const int32_t *__restrict__ perm,
             float t = bias ? bias[c + v] : 0.0f;                // A X is 0 for this row
             fill[v] = relu ? fmaxf(t, 0.0f) : t;
         }
-        store_vec_streaming<VEC>(Y + out_row * ld + c, fill, N * 4 >= ACCEL_STREAMING_MIN_BYTES);
+        store_vec<VEC, false>(Y + out_row * ld + c, fill, N * 4 >= kStreamingMinBytes);
     }
 }
 
-template <int L, int VEC, bool kWide>
+template <int L, int VEC, bool kWide, bool kShift>
 __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     const int4 *__restrict__ work, int n_units,
     const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
@@ -230,7 +203,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     __shared__ int2 stage[kWaves][kDegBound];
 
     if ((int)blockIdx.x < n_zero_groups) {
-        zero_fill_rows<VEC>(perm, Y, N, ld, n_zero_rows, bias, relu);
+        zero_fill_rows<kShift ? 1 : VEC>(perm, Y, N, ld, n_zero_rows, bias, relu);
         return;
     }
 
@@ -290,17 +263,18 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     const int k = g & (gp - 1);          // which of the row's gp groups this is
     const int rloc = g >> lg;            // which of the rows in flight
 
-    const bool streaming = N * 4 >= ACCEL_STREAMING_MIN_BYTES;
+    const bool streaming = N * 4 >= kStreamingMinBytes;
     for (int c0 = 0; c0 < N; c0 += CW) {
-        const int col = c0 + sub * VEC;
+        int col = c0 + sub * VEC;
         const bool col_ok = col < N;
+        if (kShift && col + VEC > N) col = N - VEC;   // the row's last vector ends with the row
         for (int r_it = 0; r_it < n_rows; r_it += rows_at_once) {
             const int r = r_it + rloc;
             const bool live = col_ok && r < n_rows;
             float acc[VEC];
 #pragma unroll
             for (int v = 0; v < VEC; v++) acc[v] = 0.0f;
-            if (live) gather_row<VEC, kUnroll, kWide>(st + r * d, d, k, gp, X, col, ld, acc);
+            if (live) gather_row<VEC, kUnroll, kWide, kShift>(st + r * d, d, k, gp, X, col, ld, acc);
             // add the gp partial sums of each row (all lanes take part)
             for (int m = L; m < (L << lg); m <<= 1) {
 #pragma unroll
@@ -309,8 +283,8 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
             const int64_t out_row = __shfl(my_out, r < n_rows ? r : 0);
             if (live && k == 0) {
                 if (is_long) {
-                    store_vec_streaming<VEC>(partial + (int64_t)(deg - (kDegBound + 1)) * ld + col, acc,
-                                             streaming);
+                    store_vec<VEC, kShift>(partial + (int64_t)(deg - (kDegBound + 1)) * ld + col, acc,
+                                           streaming);
                 } else {
                     if (bias) {
 #pragma unroll
@@ -320,7 +294,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 #pragma unroll
                         for (int v = 0; v < VEC; v++) acc[v] = fmaxf(acc[v], 0.0f);
                     }
-                    store_vec_streaming<VEC>(Y + out_row * ld + col, acc, streaming);
+                    store_vec<VEC, kShift>(Y + out_row * ld + col, acc, streaming);
                 }
             }
         }
@@ -332,7 +306,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
 // several wavefronts their sums meet in LDS.  Used for small matrices, where the time of
 // a launch is the longest chain of dependent gathers in one wavefront: the chain is four
 // times shorter and rows of up to one unit need no partial sums.
-template <int L, int VEC, bool kWide>
+template <int L, int VEC, bool kWide, bool kShift>
 __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
     const int4 *__restrict__ work, int n_units,
     const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
@@ -347,7 +321,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
     __shared__ float meet[kWaves][CW];
 
     if ((int)blockIdx.x < n_zero_groups) {
-        zero_fill_rows<VEC>(perm, Y, N, ld, n_zero_rows, bias, relu);
+        zero_fill_rows<kShift ? 1 : VEC>(perm, Y, N, ld, n_zero_rows, bias, relu);
         return;
     }
     const int lane = threadIdx.x & 63;
@@ -406,15 +380,16 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
     const int waves_per_row = gp > G ? gp / G : 1;   // > 1: the row's sums meet in LDS
 
     for (int c0 = 0; c0 < N; c0 += CW) {
-        const int col = c0 + sub * VEC;
+        int col = c0 + sub * VEC;
         const bool col_ok = col < N;
+        if (kShift && col + VEC > N) col = N - VEC;   // the row's last vector ends with the row
         for (int r_it = 0; r_it < n_rows; r_it += rows_at_once) {
             const int r = r_it + rloc;
             const bool live = col_ok && r < n_rows;
             float acc[VEC];
 #pragma unroll
             for (int v = 0; v < VEC; v++) acc[v] = 0.0f;
-            if (live) gather_row<VEC, kTeamUnroll, kWide>(stage + r * d, d, k, gp, X, col, ld, acc);
+            if (live) gather_row<VEC, kTeamUnroll, kWide, kShift>(stage + r * d, d, k, gp, X, col, ld, acc);
             // the row's groups inside this wavefront (all lanes take part)
             for (int m = L; m < L * in_wave; m <<= 1) {
 #pragma unroll
@@ -437,7 +412,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
             const int64_t out_row = __shfl(my_out, r < n_rows ? r : 0);
             if (live && k == 0) {
                 if (is_long)
-                    store_vec<VEC>(partial + (int64_t)(deg - (kDegBound + 1)) * ld + col, acc);
+                    store_vec<VEC, kShift>(partial + (int64_t)(deg - (kDegBound + 1)) * ld + col, acc, false);
                 else {
                     if (bias) {
 #pragma unroll
@@ -447,7 +422,7 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
 #pragma unroll
                         for (int v = 0; v < VEC; v++) acc[v] = fmaxf(acc[v], 0.0f);
                     }
-                    store_vec_streaming<VEC>(Y + out_row * ld + col, acc, N * 4 >= ACCEL_STREAMING_MIN_BYTES);
+                    store_vec<VEC, kShift>(Y + out_row * ld + col, acc, N * 4 >= kStreamingMinBytes);
                 }
             }
         }
@@ -519,37 +494,67 @@ __global__ __launch_bounds__(256) void copy_u32_kernel(uint32_t *__restrict__ ds
         dst[i] = src[i];
 }
 
-template <int VEC, bool kWide>
-int launch_for_vec(bool team, int L, dim3 grid, hipStream_t s, const int4 *work, int n_units,
-                   const int32_t *s_idx, const float *s_val, const int32_t *perm, const float *X,
-                   float *Y, float *partial, int N, int ld, int n_zero_rows, int n_zero_groups,
-                   const float *bias, int relu)
+struct LaunchArgs {
+    bool team;
+    dim3 grid;
+    hipStream_t stream;
+    const int4 *work;
+    int n_units;
+    const int32_t *s_idx;
+    const float *s_val;
+    const int32_t *perm;
+    const float *X;
+    float *Y;
+    float *partial;
+    int N, ld, n_zero_rows, n_zero_groups;
+    const float *bias;
+    int relu;
+};
+
+template <int L, int VEC, bool kWide, bool kShift>
+void launch_one(const LaunchArgs &a)
 {
-#define ACCEL_LAUNCH(LL)                                                                      \
-    case LL:                                                                                  \
-        if (team)                                                                             \
-            spmm_team_kernel<LL, VEC, kWide><<<grid, dim3(kWgThreads), 0, s>>>(                      \
-                work, n_units, s_idx, s_val, perm, X, Y, partial, N, ld, n_zero_rows,         \
-                n_zero_groups, bias, relu);                                                   \
-        else                                                                                  \
-            spmm_gather_kernel<LL, VEC, kWide><<<grid, dim3(kWgThreads), 0, s>>>(                    \
-                work, n_units, s_idx, s_val, perm, X, Y, partial, N, ld, n_zero_rows,         \
-                n_zero_groups, bias, relu);                                                   \
-        break;
+    if (a.team)
+        spmm_team_kernel<L, VEC, kWide, kShift><<<a.grid, dim3(kWgThreads), 0, a.stream>>>(
+            a.work, a.n_units, a.s_idx, a.s_val, a.perm, a.X, a.Y, a.partial, a.N, a.ld, a.n_zero_rows,
+            a.n_zero_groups, a.bias, a.relu);
+    else
+        spmm_gather_kernel<L, VEC, kWide, kShift><<<a.grid, dim3(kWgThreads), 0, a.stream>>>(
+            a.work, a.n_units, a.s_idx, a.s_val, a.perm, a.X, a.Y, a.partial, a.N, a.ld, a.n_zero_rows,
+            a.n_zero_groups, a.bias, a.relu);
+}
+
+// Lane-group widths: 1..64 lanes of one 16-byte vector each; scalar lanes only serve N < 4.
+template <int VEC, bool kWide, bool kShift>
+int launch_for_width(int L, const LaunchArgs &a)
+{
     switch (L) {
-        ACCEL_LAUNCH(1)
-        ACCEL_LAUNCH(2)
-        ACCEL_LAUNCH(4)
-        ACCEL_LAUNCH(8)
-        ACCEL_LAUNCH(16)
-        ACCEL_LAUNCH(32)
-        ACCEL_LAUNCH(64)
+    case 1: launch_one<1, VEC, kWide, kShift>(a); break;
+    case 2: launch_one<2, VEC, kWide, kShift>(a); break;
+    case 4: launch_one<4, VEC, kWide, kShift>(a); break;
     default:
+        if constexpr (VEC == 4) {
+            switch (L) {
+            case 8: launch_one<8, VEC, kWide, kShift>(a); return ACCEL_OK;
+            case 16: launch_one<16, VEC, kWide, kShift>(a); return ACCEL_OK;
+            case 32: launch_one<32, VEC, kWide, kShift>(a); return ACCEL_OK;
+            case 64: launch_one<64, VEC, kWide, kShift>(a); return ACCEL_OK;
+            }
+        }
         set_error("internal: unsupported group width %d", L);
         return ACCEL_ERR_ARG;
     }
-#undef ACCEL_LAUNCH
     return ACCEL_OK;
+}
+
+// mode: 0 = 16-byte vectors at 16-byte aligned addresses, 1 = 16-byte vectors at any
+// 4-byte aligned address with the row's last vector shifted to end with the row,
+// 2 = scalar lanes
+int launch_for_mode(int mode, bool wide, int L, const LaunchArgs &a)
+{
+    if (mode == 0) return wide ? launch_for_width<4, true, false>(L, a) : launch_for_width<4, false, false>(L, a);
+    if (mode == 1) return wide ? launch_for_width<4, true, true>(L, a) : launch_for_width<4, false, true>(L, a);
+    return wide ? launch_for_width<1, true, false>(L, a) : launch_for_width<1, false, false>(L, a);
 }
 
 }  // namespace
@@ -600,11 +605,14 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
                 hipEvent_t after_main, const float *bias, int relu, bool static_partial)
 {
     if (h->rows == 0) return ACCEL_OK;
-    // widest vector the row stride and the base pointers allow
+    // 16-byte vectors whenever a row holds one.  When N is not a multiple of 4, or X or Y
+    // is not 16-byte aligned, rows start at odd multiples of 4 bytes: the vectors are then
+    // loaded and stored at 4-byte aligned addresses, and a row's last vector is moved back
+    // so that it ends with the row (it overlaps the one before; both lanes hold the same
+    // sums for the shared columns).  Scalar lanes are left for N < 4.
     const uintptr_t align = reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Y);
-    int vec = 1;
-    if (N % 4 == 0 && align % 16 == 0) vec = 4;
-    else if (N % 2 == 0 && align % 8 == 0) vec = 2;
+    const int mode = N < 4 ? 2 : (N % 4 == 0 && align % 16 == 0) ? 0 : 1;
+    const int vec = mode == 2 ? 1 : 4;
 
     // partial sums of the pieces of split rows: the handle's buffer (allocated here when a
     // run needs more than it holds), or this GPU's static array, which is never allocated
@@ -644,16 +652,18 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     // columns have no popularity skew or the rows are very short, and a loss when N is
     // not a multiple of the panel (N = 100: 64 + 36 leaves lanes idle).
     int panel = N;
-    if (kPanel > 0 && vec == 4 && N > kPanel && N % kPanel == 0 && h->nnz >= kPanelMinNnz &&
-        h->nnz >= 16 * h->rows)
-        panel = kPanel;
+    const int want = h->plan_panel_option > 0 ? h->plan_panel_option : kPanel;
+    const bool forced = h->plan_panel_option > 0;
+    if (mode == 0 && N > want && N % want == 0 &&
+        (forced || (h->nnz >= kPanelMinNnz && h->nnz >= 16 * h->rows)))
+        panel = want;
     // operands below 4 GiB are addressed with 32-bit byte offsets (see gather_row)
     const bool wide = (uint64_t)h->cols * (uint64_t)N * 4u > 0xFFFFFFFFull;
     const int4 *wk = reinterpret_cast<const int4 *>(h->work);
     const int64_t entry_groups = h->plan_team ? h->n_units : h->n_units / kWaves;
     for (int c0 = 0; c0 < N; c0 += panel) {
         const int n = std::min(panel, N - c0);
-        int L = 1;
+        int L = 1;                                   // lanes per row: one per vector, a power of two
         while (L * vec < n && L < 64) L <<= 1;
         // zero-fill workgroups come first; their count is rounded up to a multiple of the
         // die count so that entry group i still lands on die i % 8 (surplus ones exit at once)
@@ -670,18 +680,9 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         const float *Xp = X ? X + c0 : X;
         float *Yp = Y + c0, *Pp = partial ? partial + c0 : nullptr;
         const float *bp = bias ? bias + c0 : nullptr;
-        int rc;
-#define ACCEL_DISPATCH(V)                                                                              \
-    (wide ? launch_for_vec<V, true>(h->plan_team, L, grid, stream, wk, (int)h->n_units, h->s_idx,       \
-                                    h->s_val, h->perm, Xp, Yp, Pp, n, N, (int)h->n_zero_rows,          \
-                                    (int)zero_groups, bp, relu)                                        \
-          : launch_for_vec<V, false>(h->plan_team, L, grid, stream, wk, (int)h->n_units, h->s_idx,      \
-                                     h->s_val, h->perm, Xp, Yp, Pp, n, N, (int)h->n_zero_rows,         \
-                                     (int)zero_groups, bp, relu))
-        if (vec == 4) rc = ACCEL_DISPATCH(4);
-        else if (vec == 2) rc = ACCEL_DISPATCH(2);
-        else rc = ACCEL_DISPATCH(1);
-#undef ACCEL_DISPATCH
+        const LaunchArgs la{h->plan_team, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
+                            Xp, Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu};
+        const int rc = launch_for_mode(mode, wide, L, la);
         if (rc) return rc;
     }
     if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));

@@ -81,6 +81,10 @@ class AccelSpMM:
         self._info = info
         return self
 
+    def set_panel(self, columns: int) -> None:
+        """Column-panel width of the following runs (0: automatic; see accel_set_plan_panel)."""
+        check(lib().accel_set_plan_panel(self._h, int(columns)))
+
     @property
     def info(self) -> Info:
         if self._info is None:

@@ -133,6 +133,14 @@ int accel_set_plan_groups(accel_handle *h, int groups);
  * before accel_preprocess. */
 int accel_set_plan_team(accel_handle *h, int mode);
 
+/* Column panels (no counterpart upstream, which always walks all N columns of a row
+ * at once, spmm_accel.cu:37-48): when N is a multiple of `columns` and larger, one
+ * accel_run computes Y one panel of `columns` columns at a time, all work units for
+ * the first panel before the next, so that the caches only have to hold that slice
+ * of X.  0 (the default) lets the library choose from N and the size of the matrix.
+ * Takes effect at the next accel_run; needs 16-byte aligned X and Y. */
+int accel_set_plan_panel(accel_handle *h, int columns);
+
 /* Check externally produced metadata (a .block4 file) against what
  * accel_preprocess built for this CSR; ACCEL_ERR_META if any int differs. */
 int accel_check_block4(accel_handle *h, const int32_t *block4_host, int64_t n_blocks);

@@ -13,7 +13,8 @@ from oracle import c_oracle, partition_oracle as po, spmm_oracle as so
 pytestmark = pytest.mark.gpu
 
 TOL = 1e-5
-ALL_N = [1, 2, 3, 4, 5, 6, 8, 12, 16, 17, 30, 32, 48, 60, 64, 100, 128, 130, 200, 256, 260, 300, 512, 515]
+ALL_N = [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 13, 16, 17, 30, 32, 33, 48, 50, 60, 64, 99, 100, 127, 128, 130, 200, 256,
+         257, 260, 261, 300, 512, 515]
 
 
 @pytest.fixture(scope="module", params=["workgroup units", "wavefront units"])
@@ -40,6 +41,61 @@ def test_every_column_count(gpu, mixed, N):
     assert so.check(Y, g.indptr, g.indices, g.values, X) <= TOL
     d = np.diff(g.indptr)
     assert np.array_equal(Y[d == 0], np.zeros(((d == 0).sum(), N), np.float32))   # beta = 0
+
+
+@pytest.mark.parametrize("N", [4, 5, 17, 64, 99, 259])
+def test_operands_at_any_4_byte_alignment(gpu, mixed, N):
+    """X and Y that start 4, 8 or 12 bytes past a 16-byte boundary (and rows that do so
+    because N is odd) are read and written with 16-byte accesses at those addresses; the
+    words just before and just behind Y must stay untouched."""
+    g, op = mixed
+    X = np.random.default_rng(N).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    pad = 8                                               # floats of canary on either side of Y
+    for off in (1, 2, 3):                                 # floats past the aligned start
+        hx = np.zeros(X.size + 4, np.float32)
+        hx[off:off + X.size] = X.reshape(-1)
+        dX = gpu.DeviceBuffer.from_numpy(hx)
+        dY = gpu.DeviceBuffer((g.n_rows * N + 2 * pad + 4) * 4)
+        dY.fill_u32(0x7FC00000)
+        op.run(dX.address + 4 * off, dY.address + 4 * (pad + off), N)
+        op.synchronize()
+        raw = dY.to_numpy(np.float32, (g.n_rows * N + 2 * pad + 4,))
+        Y = raw[pad + off:pad + off + g.n_rows * N].reshape(g.n_rows, N)
+        assert np.isnan(raw[:pad + off]).all() and np.isnan(raw[pad + off + g.n_rows * N:]).all()
+        assert np.isfinite(Y).all()
+        assert so.check(Y, g.indptr, g.indices, g.values, X) <= TOL
+        dX.close()
+        dY.close()
+
+
+@pytest.mark.parametrize("N", [17, 33, 50, 99, 127])
+def test_column_counts_of_upstreams_sweep_on_cfg2(gpu, N):
+    """Upstream sweeps dim 16..128 in steps of 1 (main.cu:12): three quarters of those are
+    not multiples of 4.  cfg2 is large enough for wavefront units and split rows."""
+    g = gpu.synthetic.cfg2()
+    X = gpu.synthetic.dense_operand("cfg2", g.n_cols, N)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    assert op.info.plan_team == 0 and op.info.n_split_rows > 0
+    Y = op.matmul(X)
+    R, S = c_oracle.spmm_csr_f64(g.indptr, g.indices, g.values, X)
+    assert so.scaled_error(Y, R, S) <= TOL
+    op.close()
+
+
+@pytest.mark.parametrize("N,panel", [(64, 32), (128, 32), (128, 64), (96, 32), (48, 16), (256, 128)])
+def test_column_panels(gpu, mixed, N, panel):
+    """A run cut into column panels computes the same product (a narrower panel gives a row
+    more lane groups, so the order of the additions may differ)."""
+    g, op = mixed
+    X = np.random.default_rng(N + panel).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    op.set_panel(N)                                       # one pass
+    Y1 = op.matmul(X)
+    op.set_panel(panel)
+    Yp = op.matmul(X)
+    op.set_panel(0)
+    assert np.isfinite(Yp).all()
+    assert so.check(Yp, g.indptr, g.indices, g.values, X) <= TOL
+    assert np.max(np.abs(Yp - Y1)) <= 1e-5 * np.abs(Y1).max()
 
 
 def test_workload_cfg1(gpu):
