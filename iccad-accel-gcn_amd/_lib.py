@@ -72,6 +72,8 @@ SIGNATURES = {
     "accel_set_plan_split": (C.c_int, [vp, C.c_int]),
     "accel_set_plan_team": (C.c_int, [vp, C.c_int]),
     "accel_set_plan_panel": (C.c_int, [vp, C.c_int]),
+    "accel_save_state": (C.c_int, [vp, C.c_char_p]),
+    "accel_load_state": (C.c_int, [vp, C.c_char_p]),
     "accel_check_block4": (C.c_int, [vp, i32p, C.c_int64]),
     "accel_get_info": (C.c_int, [vp, C.POINTER(Info)]),
     "accel_get_block4": (C.c_int, [vp, i32p, C.c_int64]),
@@ -79,6 +81,7 @@ SIGNATURES = {
     "accel_get_perm": (C.c_int, [vp, i32p, C.c_int64]),
     "accel_get_sorted_csr": (C.c_int, [vp, i32p, i32p, f32p]),
     "accel_run": (C.c_int, [vp, vp, vp, C.c_int32, vp]),
+    "accel_reserve": (C.c_int, [vp, C.c_int32]),
     "accel_run_static": (C.c_int, [vp, vp, vp, C.c_int32, vp]),
     "accel_run_epilogue": (C.c_int, [vp, vp, vp, C.c_int32, vp, C.c_int, vp]),
     "accel_time": (C.c_int, [vp, vp, vp, C.c_int32, C.c_int, C.c_int, f32p, f32p, vp]),
@@ -133,6 +136,31 @@ def ptr(a, ctype=None):
     if hasattr(a, "data_ptr"):
         return C.c_void_p(int(a.data_ptr()))
     return C.c_void_p(int(a))
+
+
+def dev_ptr(a, need_bytes: int, name: str):
+    """Address of a dense operand on the device.  A numpy array is host memory and is
+    refused here (the kernels would fault on it); where the object tells its size, that
+    size must cover ``need_bytes``.  Raw integer addresses are passed through: the
+    library asks the HIP runtime about them."""
+    if a is None:
+        return None
+    if isinstance(a, np.ndarray):
+        raise AccelError(ERR_ARG, f"{name} is a numpy array (host memory); pass a DeviceBuffer, an object "
+                                  "with data_ptr() on the GPU, or a device address")
+    have = None
+    if isinstance(a, DeviceBuffer):
+        if not a.address:
+            raise AccelError(ERR_ARG, f"{name} is a closed DeviceBuffer")
+        have = a.nbytes
+    elif hasattr(a, "data_ptr"):
+        if getattr(a, "is_cuda", True) is False:
+            raise AccelError(ERR_ARG, f"{name} is a host tensor; move it to the GPU first")
+        if hasattr(a, "numel") and hasattr(a, "element_size"):
+            have = int(a.numel()) * int(a.element_size())
+    if have is not None and have < need_bytes:
+        raise AccelError(ERR_ARG, f"{name} holds {have} bytes, {need_bytes} needed")
+    return ptr(a)
 
 
 class DeviceBuffer:

@@ -17,7 +17,7 @@ CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB = LIB_DIR / "libaccelgcn.so"
 BIN_DIR = PKG / "bin"
-SOURCES = ["capi.hip", "preprocess.hip", "spmm.hip", "spmm_accel.cpp"]
+SOURCES = ["capi.hip", "preprocess.hip", "spmm.hip", "state.hip", "spmm_accel.cpp"]
 ARCH = "gfx950"
 
 
@@ -35,17 +35,16 @@ def compile_flags():
             f"-I{ROOT / 'include'}", f"-I{CSRC}"]
 
 
-def build(verbose: bool = False, extra_flags=(), out: Path | None = None) -> Path:
-    """Compile and link; ``extra_flags`` (e.g. -DACCEL_UNROLL=8) and ``out`` let a
-    tuning variant be built next to the default library."""
+def build(verbose: bool = False) -> Path:
+    """Compile every source and link lib/libaccelgcn.so, then the two programs in bin/
+    and the comparison-baselines library."""
     LIB_DIR.mkdir(exist_ok=True)
-    out = Path(out) if out else LIB
-    out.parent.mkdir(parents=True, exist_ok=True)
+    out = LIB
     objs = []
     procs = []
     for src in SOURCES:
         obj = out.parent / (out.stem + "." + src + ".o")
-        cmd = [hipcc(), *compile_flags(), *extra_flags, "-c", str(CSRC / src), "-o", str(obj)]
+        cmd = [hipcc(), *compile_flags(), "-c", str(CSRC / src), "-o", str(obj)]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -65,9 +64,8 @@ def build(verbose: bool = False, extra_flags=(), out: Path | None = None) -> Pat
     os.replace(tmp, out)
     for o in objs:
         os.unlink(o)
-    if out == LIB:
-        build_cli(verbose)
-        build_baselines(verbose)
+    build_cli(verbose)
+    build_baselines(verbose)
     return out
 
 
@@ -88,17 +86,19 @@ def build_baselines(verbose: bool = False) -> Path:
 
 
 def build_cli(verbose: bool = False) -> Path:
-    """bin/spmm_test: the command-line harness (counterpart of upstream's main.cu)."""
+    """bin/spmm_test: the command-line harness (counterpart of upstream's main.cu);
+    bin/operator_check: error paths of the C++ operator, run by the tests."""
     BIN_DIR.mkdir(exist_ok=True)
-    exe = BIN_DIR / "spmm_test"
-    cmd = [hipcc(), *compile_flags(), str(CSRC / "spmm_test.cpp"), "-o", str(exe),
-           f"-L{LIB_DIR}", "-laccelgcn", "-Wl,-rpath,$ORIGIN/../lib"]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("hipcc failed for spmm_test.cpp:\n" + r.stdout)
-    return exe
+    for name in ("spmm_test", "operator_check"):
+        exe = BIN_DIR / name
+        cmd = [hipcc(), *compile_flags(), str(CSRC / f"{name}.cpp"), "-o", str(exe),
+               f"-L{LIB_DIR}", "-laccelgcn", "-Wl,-rpath,$ORIGIN/../lib"]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {name}.cpp:\n" + r.stdout)
+    return BIN_DIR / "spmm_test"
 
 
 if __name__ == "__main__":

@@ -26,7 +26,7 @@ void clear_error() { g_error.clear(); }
 int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
                           int32_t **block4_dev, int64_t *n_blocks);
 
-static void release_products(accel_handle *h)
+void release_products(accel_handle *h)
 {
     if (h->perm) (void)hipFree(h->perm);
     if (h->s_indptr) (void)hipFree(h->s_indptr);
@@ -38,6 +38,8 @@ static void release_products(accel_handle *h)
     if (h->long_slot) (void)hipFree(h->long_slot);
     if (h->block4) (void)hipFree(h->block4);
     if (h->partial) (void)hipFree(h->partial);
+    if (h->partial_done) (void)hipEventDestroy(h->partial_done);
+    h->partial_done = nullptr; h->partial_stream = nullptr; h->partial_in_use = false;
     h->perm = nullptr; h->s_indptr = nullptr; h->s_idx = nullptr; h->s_val = nullptr;
     h->work = nullptr; h->long_slot = nullptr; h->block4 = nullptr; h->partial = nullptr;
     h->n_units = h->n_long_units = 0;
@@ -55,6 +57,52 @@ static int need_gpu()
         return ACCEL_ERR_HIP;
     }
     return ACCEL_OK;
+}
+
+// A dense operand must be memory the GPU can read: a host address handed to a kernel is a
+// memory fault, not an error code.  The runtime is asked what the address is and, where it
+// knows the allocation, whether `bytes` fit behind it.  Each (address, size) that passed is
+// remembered, so the check costs nothing in a loop over the same buffers.
+static int check_operand(accel_handle *h, const void *p, size_t bytes, const char *fn, const char *name)
+{
+    if (!p || bytes == 0) return ACCEL_OK;
+    for (const auto &c : h->checked)
+        if (c.p == p && c.bytes >= bytes) return ACCEL_OK;
+    hipPointerAttribute_t at;
+    if (hipPointerGetAttributes(&at, p) != hipSuccess || at.type == hipMemoryTypeUnregistered) {
+        (void)hipGetLastError();
+        set_error("%s: %s (%p) is not memory the GPU can access (a host array? copy it to the device first)",
+                  fn, name, p);
+        return ACCEL_ERR_ARG;
+    }
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(&base, &size, const_cast<void *>(p)) == hipSuccess && base) {
+        const size_t off = (size_t)(static_cast<const char *>(p) - static_cast<const char *>(base));
+        if (off > size || size - off < bytes) {
+            set_error("%s: %s needs %zu bytes, its allocation holds %zu from that address", fn, name, bytes,
+                      off > size ? (size_t)0 : size - off);
+            return ACCEL_ERR_ARG;
+        }
+    } else {
+        (void)hipGetLastError();
+    }
+    h->checked[h->checked_next] = {p, bytes};
+    h->checked_next = (h->checked_next + 1) % 4;
+    return ACCEL_OK;
+}
+
+// argument checks shared by the run entry points
+static int check_run(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias, const char *fn)
+{
+    if (!h) { set_error("%s: null handle", fn); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("%s: call accel_preprocess first", fn); return ACCEL_ERR_STATE; }
+    if (N <= 0) { set_error("%s: N must be positive, got %d", fn, N); return ACCEL_ERR_ARG; }
+    if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("%s: null dense operand", fn); return ACCEL_ERR_ARG; }
+    if (h->rows == 0) return ACCEL_OK;
+    if (int rc = check_operand(h, X, (size_t)h->cols * (size_t)N * sizeof(float), fn, "X")) return rc;
+    if (int rc = check_operand(h, Y, (size_t)h->rows * (size_t)N * sizeof(float), fn, "Y")) return rc;
+    return check_operand(h, bias, (size_t)N * sizeof(float), fn, "bias");
 }
 
 }  // namespace accel
@@ -567,20 +615,23 @@ int accel_partition_gpu(const int32_t *indptr, int64_t rows, int32_t *block4_out
 int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream)
 {
     clear_error();
-    if (!h) { set_error("accel_run: null handle"); return ACCEL_ERR_ARG; }
-    if (!h->ready) { set_error("accel_run: call accel_preprocess first"); return ACCEL_ERR_STATE; }
-    if (N <= 0) { set_error("accel_run: N must be positive, got %d", N); return ACCEL_ERR_ARG; }
-    if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("accel_run: null dense operand"); return ACCEL_ERR_ARG; }
+    if (int rc = check_run(h, X, Y, N, nullptr, "accel_run")) return rc;
     return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr);
+}
+
+int accel_reserve(accel_handle *h, int32_t max_N)
+{
+    clear_error();
+    if (!h) { set_error("accel_reserve: null handle"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_reserve: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (max_N <= 0) { set_error("accel_reserve: N must be positive, got %d", max_N); return ACCEL_ERR_ARG; }
+    return reserve_partial(h, (size_t)h->n_long_units * (size_t)max_N);
 }
 
 int accel_run_static(accel_handle *h, const float *X, float *Y, int32_t N, void *stream)
 {
     clear_error();
-    if (!h) { set_error("accel_run_static: null handle"); return ACCEL_ERR_ARG; }
-    if (!h->ready) { set_error("accel_run_static: call accel_preprocess first"); return ACCEL_ERR_STATE; }
-    if (N <= 0) { set_error("accel_run_static: N must be positive, got %d", N); return ACCEL_ERR_ARG; }
-    if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("accel_run_static: null dense operand"); return ACCEL_ERR_ARG; }
+    if (int rc = check_run(h, X, Y, N, nullptr, "accel_run_static")) return rc;
     return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, nullptr, 0, true);
 }
 
@@ -588,10 +639,7 @@ int accel_run_epilogue(accel_handle *h, const float *X, float *Y, int32_t N, con
                        int flags, void *stream)
 {
     clear_error();
-    if (!h) { set_error("accel_run_epilogue: null handle"); return ACCEL_ERR_ARG; }
-    if (!h->ready) { set_error("accel_run_epilogue: call accel_preprocess first"); return ACCEL_ERR_STATE; }
-    if (N <= 0) { set_error("accel_run_epilogue: N must be positive, got %d", N); return ACCEL_ERR_ARG; }
-    if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("accel_run_epilogue: null dense operand"); return ACCEL_ERR_ARG; }
+    if (int rc = check_run(h, X, Y, N, bias, "accel_run_epilogue")) return rc;
     if (flags & ~ACCEL_EPILOGUE_RELU) { set_error("accel_run_epilogue: unknown flags %d", flags); return ACCEL_ERR_ARG; }
     return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, bias,
                        (flags & ACCEL_EPILOGUE_RELU) ? 1 : 0);
@@ -601,10 +649,8 @@ int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup,
                float *ms_total, float *ms_main, void *stream)
 {
     clear_error();
-    if (!h) { set_error("accel_time: null handle"); return ACCEL_ERR_ARG; }
-    if (!h->ready) { set_error("accel_time: call accel_preprocess first"); return ACCEL_ERR_STATE; }
-    if (N <= 0 || warmup < 0 || iters < 0) { set_error("accel_time: bad N/warmup/iters"); return ACCEL_ERR_ARG; }
-    if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("accel_time: null dense operand"); return ACCEL_ERR_ARG; }
+    if (warmup < 0 || iters < 0) { set_error("accel_time: bad warmup/iters"); return ACCEL_ERR_ARG; }
+    if (int rc = check_run(h, X, Y, N, nullptr, "accel_time")) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     for (int i = 0; i < warmup; i++)
         if (int rc = spmm_launch(h, X, Y, N, s, nullptr)) return rc;

@@ -118,15 +118,27 @@ struct accel_handle {
     // scratch for the partial sums of long-row segments: [n_long_blocks * N]
     float *partial = nullptr;
     size_t partial_floats = 0;
+    // which stream used `partial` last, and an event recorded behind that run
+    hipStream_t partial_stream = nullptr;
+    hipEvent_t partial_done = nullptr;
+    bool partial_in_use = false;
+    // dense operands already checked (address, bytes needed): see check_operand in capi.hip
+    struct Checked { const void *p = nullptr; size_t bytes = 0; } checked[4];
+    int checked_next = 0;
 };
 
 namespace accel {
 // preprocess.hip
 int preprocess_device(accel_handle *h);
+int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s);
+int hash_words_device(const void *words_dev, int64_t n, uint64_t seed, uint64_t *out_dev, hipStream_t s);
+// capi.hip
+void release_products(accel_handle *h);
 // spmm.hip
 int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
                 hipEvent_t after_main, const float *bias = nullptr, int relu = 0,
                 bool static_partial = false);
+int reserve_partial(accel_handle *h, size_t floats);
 int fill_u32(void *dst, uint32_t v, size_t n, hipStream_t s);
 int copy_u32(void *dst, const void *src, size_t n, hipStream_t s);
 }  // namespace accel

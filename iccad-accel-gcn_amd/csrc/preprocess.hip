@@ -503,7 +503,8 @@ __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
 // Split rows: the row's non-zeros are written to the sorted CSR grouped by
 // col_group(column, row_groups(degree)), stably inside each group, so that a
 // work unit of such a row touches rows of X that belong to one column group.
-// One workgroup per split row; counts[lr*64 + g] receives the size of each group.
+// One workgroup per split row; counts[lr*64 + g] receives the size of each group
+// (counts may be null).
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
     const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
@@ -528,7 +529,7 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
         int b = 0;
         for (int g = 0; g < (int)threadIdx.x; g++) b += cnt[g];
         base[threadIdx.x] = b;
-        counts[(int64_t)blockIdx.x * kMaxGroups + threadIdx.x] = cnt[threadIdx.x];
+        if (counts) counts[(int64_t)blockIdx.x * kMaxGroups + threadIdx.x] = cnt[threadIdx.x];
     }
     __syncthreads();
     int flip = 0;
@@ -1169,6 +1170,84 @@ static int choose_plan_split(int64_t rows, int64_t nnz, bool team)
     (void)rows;
     (void)nnz;
     return team ? kDegBound : ACCEL_PLAN_SPLIT;        // workgroup units: rows up to one unit stay whole
+}
+
+// 64-bit content hash of n 4-byte words: the sum over i of mix(i, word i) modulo 2^64,
+// so the order of the additions does not matter.  *out must be zero on entry.
+__device__ __forceinline__ uint64_t mix64(uint64_t x)
+{
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+__global__ __launch_bounds__(kThreads) void hash_words_kernel(const uint32_t *__restrict__ a, int64_t n,
+                                                              uint64_t seed,
+                                                              unsigned long long *__restrict__ out)
+{
+    __shared__ unsigned long long part[kThreads / 64];
+    uint64_t acc = 0;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads)
+        acc += mix64((((uint64_t)i << 32) | a[i]) ^ seed);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor((unsigned long long)acc, off);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int q = 1; q < kThreads / 64; q++) acc += part[q];
+        atomicAdd(out, (unsigned long long)acc);
+    }
+}
+
+int hash_words_device(const void *words_dev, int64_t n, uint64_t seed, uint64_t *out_dev, hipStream_t s)
+{
+    if (n <= 0) return ACCEL_OK;
+    const unsigned g = (unsigned)std::min<int64_t>((n + kThreads - 1) / kThreads, 4096);
+    hash_words_kernel<<<dim3(g), dim3(kThreads), 0, s>>>(static_cast<const uint32_t *>(words_dev), n, seed,
+                                                         reinterpret_cast<unsigned long long *>(out_dev));
+    ACCEL_HIP(hipGetLastError());
+    return ACCEL_OK;
+}
+
+// The degree-sorted copy of the CSR from the caller's arrays, perm, s_indptr and the
+// plan's split threshold: what accel_preprocess builds between the sort and the
+// partition.  Used when those products come from a saved state.  Needs h->perm (or
+// identity_perm), h->s_indptr, h->n_split_rows and h->plan_groups; sets s_idx, s_val,
+// owns_sorted.  nnz_short = non-zeros of the rows that are not split.
+int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s)
+{
+    const int64_t rows = h->rows, nnz = h->nnz, n_long = h->n_split_rows, first_long = rows - n_long;
+    if (h->identity_perm && n_long == 0) {
+        h->s_idx = h->idx;
+        h->s_val = h->val;
+        h->owns_sorted = false;
+        return ACCEL_OK;
+    }
+    DevBuf sidx, sval;
+    int rc;
+    if ((rc = sidx.alloc(sizeof(int32_t) * (size_t)nnz))) return rc;
+    if ((rc = sval.alloc(sizeof(float) * (size_t)nnz))) return rc;
+    if (nnz_short > 0) {
+        if (h->identity_perm) {
+            ACCEL_HIP(hipMemcpyAsync(sidx.p, h->idx, sizeof(int32_t) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
+            ACCEL_HIP(hipMemcpyAsync(sval.p, h->val, sizeof(float) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
+        } else {
+            permute_csr_kernel<<<dim3((unsigned)((nnz_short + kPermuteTile - 1) / kPermuteTile)), dim3(kThreads), 0, s>>>(
+                h->indptr, h->idx, h->val, h->perm, h->s_indptr, rows, nnz_short, sidx.as<int32_t>(),
+                sval.as<float>());
+        }
+    }
+    if (n_long > 0)
+        group_long_rows_kernel<<<dim3((unsigned)n_long), dim3(kThreads), 0, s>>>(
+            h->indptr, h->idx, h->val, h->perm, h->s_indptr, first_long, h->plan_groups,
+            sidx.as<int32_t>(), sval.as<float>(), nullptr);
+    ACCEL_HIP(hipGetLastError());
+    ACCEL_HIP(hipStreamSynchronize(s));
+    h->s_idx = static_cast<int32_t *>(sidx.release());
+    h->s_val = static_cast<float *>(sval.release());
+    h->owns_sorted = true;
+    return ACCEL_OK;
 }
 
 int preprocess_device(accel_handle *h)

@@ -601,6 +601,24 @@ static int static_scratch_address(float **out)
     return ACCEL_OK;
 }
 
+// Grows the handle's partial-sum buffer to `floats` (never shrinks).  The old buffer is
+// freed: graphs captured with it must be captured again.
+int reserve_partial(accel_handle *h, size_t floats)
+{
+    if (h->partial_floats >= floats) return ACCEL_OK;
+    if (h->partial_in_use) (void)hipEventSynchronize(h->partial_done);   // nobody reads the old one
+    if (h->partial) (void)hipFree(h->partial);
+    h->partial = nullptr;
+    h->partial_floats = 0;
+    if (hipMalloc(reinterpret_cast<void **>(&h->partial), floats * sizeof(float)) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("device allocation of %zu bytes for long-row partial sums failed", floats * sizeof(float));
+        return ACCEL_ERR_ALLOC;
+    }
+    h->partial_floats = floats;
+    return ACCEL_OK;
+}
+
 int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
                 hipEvent_t after_main, const float *bias, int relu, bool static_partial)
 {
@@ -617,6 +635,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     // partial sums of the pieces of split rows: the handle's buffer (allocated here when a
     // run needs more than it holds), or this GPU's static array, which is never allocated
     float *partial = h->partial;
+    bool guard_partial = false;
     if (static_partial) {
         partial = nullptr;
         const size_t need = (size_t)h->n_long_units * (size_t)N;
@@ -629,20 +648,31 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         if (need > 0)
             if (int rc = static_scratch_address(&partial)) return rc;
     } else if (h->n_long_units > 0) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        (void)hipStreamIsCapturing(stream, &cap);
+        if (hipGetLastError() != hipSuccess) cap = hipStreamCaptureStatusNone;
+        const bool capturing = cap != hipStreamCaptureStatusNone;
+        // The buffer is shared by all runs of this handle: a run on another stream may only
+        // start once the previous one has finished (runs queued on one stream are ordered).
+        if (h->partial_in_use && stream != h->partial_stream && !capturing &&
+            hipEventQuery(h->partial_done) == hipErrorNotReady) {
+            (void)hipGetLastError();
+            set_error("this handle is still running on another stream; its partial-sum buffer is "
+                      "shared: wait for that run, or use one handle per stream");
+            return ACCEL_ERR_STATE;
+        }
+        (void)hipGetLastError();
         const size_t need = (size_t)h->n_long_units * (size_t)N;
         if (h->partial_floats < need) {
-            if (h->partial) (void)hipFree(h->partial);
-            h->partial = nullptr;
-            h->partial_floats = 0;
-            if (hipMalloc(reinterpret_cast<void **>(&h->partial), need * sizeof(float)) != hipSuccess) {
-                (void)hipGetLastError();
-                set_error("device allocation of %zu bytes for long-row partial sums failed",
-                          need * sizeof(float));
-                return ACCEL_ERR_ALLOC;
+            if (capturing) {
+                set_error("the partial-sum buffer has to grow for N = %d and the stream is capturing: "
+                          "call accel_reserve(h, N) before the capture", N);
+                return ACCEL_ERR_STATE;
             }
-            h->partial_floats = need;
+            if (int rc = reserve_partial(h, need)) return rc;
         }
         partial = h->partial;
+        guard_partial = !capturing;
     }
     // Wide operands are computed one column panel at a time (all units for the first
     // panel, then all units for the next): a panel's slice of X is what the L2s have
@@ -697,6 +727,12 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
             n_split, Y, N, bias, relu);
     }
     ACCEL_HIP(hipGetLastError());
+    if (guard_partial) {
+        if (!h->partial_done) ACCEL_HIP(hipEventCreateWithFlags(&h->partial_done, hipEventDisableTiming));
+        ACCEL_HIP(hipEventRecord(h->partial_done, stream));
+        h->partial_stream = stream;
+        h->partial_in_use = true;
+    }
     return ACCEL_OK;
 }
 

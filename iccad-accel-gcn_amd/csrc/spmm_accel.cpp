@@ -15,7 +15,17 @@ bool SPMM_ACCEL::preprocess()
     if (h) return true;
     err.clear();
     int rc = accel_create(ptr, idx, val, num_v, num_v, num_e, ACCEL_PTR_DEVICE, &h);
-    if (!rc) rc = accel_preprocess(h);
+    if (!rc) {
+        // A state saved by an earlier run takes the place of the preprocessing, as upstream
+        // loads its metadata file instead of recomputing (spmm_accel.cu:122).  A state that
+        // is missing, damaged or belongs to another CSR is a stale cache entry, not an error.
+        const std::string state = meta_dir + _graph + ".accelstate";
+        from_state = accel_load_state(h, state.c_str()) == ACCEL_OK;
+        if (!from_state) {
+            rc = accel_preprocess(h);
+            if (!rc && save_state) (void)accel_save_state(h, state.c_str());   // best effort
+        }
+    }
     accel_info info{};
     if (!rc) rc = accel_get_info(h, &info);
     if (!rc) {
@@ -44,13 +54,14 @@ bool SPMM_ACCEL::preprocess()
 
 void SPMM_ACCEL::run(int dim)
 {
-    if (!h) return;
+    if (!h || !err.empty()) return;   // nothing is launched after a failure
     if (accel_run(h, vin, vout, dim, nullptr) != ACCEL_OK) err = accel_last_error();
 }
 
 double SPMM_ACCEL::do_test(bool timing, int dim)
 {
     if (!preprocess()) return -1.0;
+    err.clear();                      // a failure of an earlier call does not stick
     const double t = timing_body(timing, dim);
     return err.empty() ? t : -1.0;
 }

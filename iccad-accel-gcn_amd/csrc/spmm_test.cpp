@@ -4,6 +4,9 @@
 //   spmm_test <graph> <dim>      check against a host CSR loop, then time (main.cu:186-194)
 //   spmm_test                    time every <graphs>/*.config for dim 16..128 (main.cu:195-219)
 //   options: --graphs DIR (default ../graphs/)  --meta DIR (default ../block_level_meta/)
+//            --save-state   write <meta>/<graph>.accelstate after preprocessing; a later run
+//                           loads it instead of preprocessing (as upstream loads its .block4,
+//                           spmm_accel.cu:122) and says so on stderr
 //
 // Input files, as upstream reads them (main.cu:62-63, data.h:7-21): <graph>.new_indptr and
 // <graph>.new_indices, raw little-endian int32.  Values are all 1 and vin ~ U[0,1) from
@@ -30,6 +33,7 @@ std::string base_dir = "../graphs/";
 std::string meta_dir = "../block_level_meta/";
 int dim_min = 16, dim_max = 128, interval = 1;
 int total_file_cnt = 0, current_file_cnt = 0;
+bool save_state = false;
 
 template <class T>
 bool read_managed(const std::string &path, T **arr, int64_t *count)
@@ -110,6 +114,8 @@ int test_graph(const std::string &graph, int spec_dim, bool checking, bool timin
 
     SPMM_ACCEL accel(graph, indptr, indices, val, vin, vout, v_num, e_num, hi);
     accel.set_meta_dir(meta_dir);
+    accel.set_save_state(save_state);
+    bool said = false;
     int rc = 0;
     std::vector<float> ref;
     for (int dim = lo; dim <= hi && rc == 0; dim += interval) {
@@ -120,6 +126,8 @@ int test_graph(const std::string &graph, int spec_dim, bool checking, bool timin
                 rc = 1;
                 break;
             }
+            if (!said && accel.loaded_from_state()) std::cerr << "accel: preprocessing loaded from saved state" << std::endl;
+            said = true;
             ref.resize((size_t)v_num * dim);
             host_reference(indptr, indices, val, vin, ref.data(), v_num, dim);
             bool has_err = false;
@@ -156,6 +164,7 @@ int main(int argc, char *argv[])
         const std::string a = argv[i];
         if (a == "--graphs" && i + 1 < argc) base_dir = argv[++i];
         else if (a == "--meta" && i + 1 < argc) meta_dir = argv[++i];
+        else if (a == "--save-state") save_state = true;
         else pos.push_back(a);
     }
     if (!base_dir.empty() && base_dir.back() != '/') base_dir += '/';

@@ -81,6 +81,20 @@ class AccelSpMM:
         self._info = info
         return self
 
+    def save_state(self, path) -> None:
+        """Write what preprocess() built (block4, permutation, launch plan) to ``path``."""
+        self.info
+        check(lib().accel_save_state(self._h, str(path).encode()))
+
+    def load_state(self, path) -> "AccelSpMM":
+        """Take the place of preprocess(): load a state saved for the same CSR.
+        Raises AccelError (ERR_META) if the file belongs to another CSR or is damaged."""
+        check(lib().accel_load_state(self._h, str(path).encode()))
+        info = Info()
+        check(lib().accel_get_info(self._h, C.byref(info)))
+        self._info = info
+        return self
+
     def set_panel(self, columns: int) -> None:
         """Column-panel width of the following runs (0: automatic; see accel_set_plan_panel)."""
         check(lib().accel_set_plan_panel(self._h, int(columns)))
@@ -126,19 +140,35 @@ class AccelSpMM:
         check(lib().accel_check_block4(self._h, ptr(b, C.c_int32), b.size // 4))
 
     # -- run ----------------------------------------------------------------
+    def _operands(self, X, Y, N, bias=None):
+        """Device addresses of the dense operands, after the checks the host can make."""
+        N = int(N)
+        if N <= 0:
+            raise AccelError(_lib.ERR_ARG, f"N must be positive, got {N}")
+        return (_lib.dev_ptr(X, self.n_cols * N * 4, "X"), _lib.dev_ptr(Y, self.n_rows * N * 4, "Y"),
+                _lib.dev_ptr(bias, N * 4, "bias"))
+
     def run(self, X, Y, N: int, stream=None) -> None:
         """One asynchronous launch; X, Y are device buffers."""
-        check(lib().accel_run(self._h, ptr(X), ptr(Y), int(N), ptr(stream)))
+        x, y, _ = self._operands(X, Y, N)
+        check(lib().accel_run(self._h, x, y, int(N), ptr(stream)))
+
+    def reserve(self, max_N: int) -> None:
+        """Allocate the partial-sum buffer for every N up to ``max_N`` now, so that no later
+        run allocates (see accel_reserve)."""
+        check(lib().accel_reserve(self._h, int(max_N)))
 
     def run_static(self, X, Y, N: int, stream=None) -> None:
         """``run`` without any device allocation: the partial sums of split rows go to
         the library's static scratch array (ACCEL_STATIC_SCRATCH_BYTES per GPU) and a
         matrix that needs more at this N is refused (see accel_run_static)."""
-        check(lib().accel_run_static(self._h, ptr(X), ptr(Y), int(N), ptr(stream)))
+        x, y, _ = self._operands(X, Y, N)
+        check(lib().accel_run_static(self._h, x, y, int(N), ptr(stream)))
 
     def run_epilogue(self, X, Y, N: int, bias=None, relu=False, stream=None) -> None:
         """Y = act(A X + bias) in one launch; bias is a device buffer of N floats or None."""
-        check(lib().accel_run_epilogue(self._h, ptr(X), ptr(Y), int(N), ptr(bias),
+        x, y, b = self._operands(X, Y, N, bias)
+        check(lib().accel_run_epilogue(self._h, x, y, int(N), b,
                                        _lib.EPILOGUE_RELU if relu else 0, ptr(stream)))
 
     def synchronize(self, stream=None) -> None:
@@ -167,7 +197,8 @@ class AccelSpMM:
         where the extra event is a visible part of the total."""
         tot = np.zeros(iters, dtype=np.float32)
         main = np.zeros(iters, dtype=np.float32)
-        check(lib().accel_time(self._h, ptr(X), ptr(Y), int(N), warmup, iters,
+        x, y, _ = self._operands(X, Y, N)
+        check(lib().accel_time(self._h, x, y, int(N), warmup, iters,
                                ptr(tot, C.c_float), ptr(main, C.c_float) if split else None, ptr(stream)))
         return tot, main
 
@@ -198,13 +229,31 @@ class SpmmAccel:
         self.vin, self.vout = vin, vout
         self.num_v, self.num_e, self.dim = int(num_v), int(num_e), int(dim)
         self.meta_dir = Path(meta_dir)
+        self.save_state = False        # True: write <meta_dir>/<graph>.accelstate after preprocessing
+        self.state_loaded = False
         self._op = AccelSpMM(ptr_, idx, val, self.num_v, device=True, n_rows=self.num_v, nnz=self.num_e)
         self._ready = False
 
     def _preprocess(self):
         if self._ready:
             return
-        self._op.preprocess()
+        # the saved state of an earlier run takes the place of the preprocessing, as
+        # upstream's operator loads its metadata file (spmm_accel.cu:122); a state that
+        # does not belong to this CSR is a stale cache entry, not an error
+        state = self.meta_dir / f"{self._graph}.accelstate"
+        loaded = False
+        if state.exists():
+            try:
+                self._op.load_state(state)
+                loaded = True
+            except AccelError as e:
+                if e.status not in (_lib.ERR_META, _lib.ERR_IO):
+                    raise
+        if not loaded:
+            self._op.preprocess()
+            if self.save_state and self.meta_dir.is_dir():
+                self._op.save_state(state)
+        self.state_loaded = loaded
         meta = self.meta_dir / f"{self._graph}.block4"
         if meta.exists():      # a stale file must not pass silently (spmm_accel.cu:122 trusts it blindly)
             self._op.check_block4(np.fromfile(meta, dtype="<i4"))

@@ -133,6 +133,22 @@ int accel_set_plan_groups(accel_handle *h, int groups);
  * before accel_preprocess. */
 int accel_set_plan_team(accel_handle *h, int mode);
 
+/* Saved preprocessing state.  Upstream persists its preprocessing as a file
+ * (block_level_partition.py:105-106 writes <graph>.block4) and its operator loads
+ * that file instead of recomputing (spmm_accel.cu:122).  accel_save_state writes
+ * what accel_preprocess built for this handle: the block4 metadata, the degree-sort
+ * permutation, the sorted indptr, the launch plan and the partial-sum slots (not the
+ * sorted copy of the non-zeros, which is regathered on load).  accel_load_state takes
+ * the place of accel_preprocess on a handle created on the same CSR: the file is
+ * keyed by content hashes of indptr and idx, computed on the GPU; a file saved for
+ * another CSR, by another library version, or damaged (every stored array carries
+ * a hash) gives ACCEL_ERR_META and leaves the handle un-preprocessed, a missing or
+ * short file ACCEL_ERR_IO.  After a successful load the handle behaves exactly as
+ * after accel_preprocess with the options the state was saved with (the results of
+ * accel_run are the same bits); accel_info.preprocess_ms is the time of the load. */
+int accel_save_state(const accel_handle *h, const char *path);
+int accel_load_state(accel_handle *h, const char *path);
+
 /* Column panels (no counterpart upstream, which always walks all N columns of a row
  * at once, spmm_accel.cu:37-48): when N is a multiple of `columns` and larger, one
  * accel_run computes Y one panel of `columns` columns at a time, all work units for
@@ -193,7 +209,12 @@ int accel_get_plan(const accel_handle *h, int32_t *out, int64_t cap_units, int64
  * spmm_accel.cu:84,97).  X has cols(A) rows, Y has rows(A) rows, both with
  * leading dimension N (spmm_accel.cu:75,84 index row*feat_in+lane).  Rows of Y
  * are in the caller's original row order.  Asynchronous on `stream` (a
- * hipStream_t, NULL = default stream); X and Y are device pointers. */
+ * hipStream_t, NULL = default stream); X and Y are device pointers: an address the
+ * GPU cannot read, or an allocation too small for cols x N (X) or rows x N (Y) floats,
+ * is refused with ACCEL_ERR_ARG where the runtime can tell.  One handle runs on one
+ * stream at a time: its partial-sum buffer is shared, and a run on a second stream
+ * while the previous one is still in flight returns ACCEL_ERR_STATE (runs queued on
+ * the same stream are ordered and fine; distinct handles are independent). */
 int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream);
 
 /* run with the rest of a GCN layer fused into the store: Y = act(A X + bias).
@@ -204,6 +225,16 @@ int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream
 #define ACCEL_EPILOGUE_RELU 1
 int accel_run_epilogue(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias,
                        int flags, void *stream);
+
+/* accel_run keeps the partial sums of split rows (pieces x N floats) in a buffer of the
+ * handle.  It is allocated by the first accel_run with a given N and replaced by a larger
+ * one when a later run brings a larger N; a HIP graph captured with the old buffer must
+ * then be captured again.  accel_reserve allocates it for every N up to max_N at once, so
+ * that no later accel_run with N <= max_N allocates or frees: call it before capturing a
+ * graph or entering a loop that must not allocate (a run that would have to grow the
+ * buffer while its stream is capturing fails with ACCEL_ERR_STATE).  No counterpart
+ * upstream, whose kernel adds split rows up with atomicAdd (spmm_accel.cu:84,97). */
+int accel_reserve(accel_handle *h, int32_t max_N);
 
 /* accel_run for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no

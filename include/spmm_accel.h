@@ -13,6 +13,7 @@
  * that file exists it is compared with the GPU-built metadata and a mismatch is
  * an error (do_test returns -1), so a stale file cannot silently mis-index.
  * run(dim): one asynchronous launch; vout = A * vin with leading dimension dim.
+ * After a launch has failed, run() launches nothing more and do_test returns -1.
  *
  * Differences from upstream that a caller can observe:
  *   - vout is overwritten (beta = 0), zero-degree rows become 0; upstream
@@ -36,6 +37,13 @@ public:
     double do_test(bool timing, int dim) override;
     /* Directory searched for "<graph>.block4" (default: upstream's relative path). */
     void set_meta_dir(const std::string &dir) { meta_dir = dir; }
+    /* Preprocessing cache, the counterpart of upstream loading its metadata file on every
+     * do_test (spmm_accel.cu:122): "<meta_dir><graph>.accelstate", written by
+     * accel_save_state, is loaded instead of preprocessing when it belongs to this CSR
+     * (keyed by content hashes); otherwise the preprocessing runs and, after
+     * set_save_state(true), writes that file.  loaded_from_state() tells which happened. */
+    void set_save_state(bool on) { save_state = on; }
+    bool loaded_from_state() const { return from_state; }
     /* Text of the last error ("" if none). */
     const std::string &error() const { return err; }
     /* Number of block4 entries after preprocessing. */
@@ -48,5 +56,6 @@ protected:
     std::string meta_dir = "../block_level_meta/";
     std::string err;
     long long n_blocks = 0;
+    bool save_state = false, from_state = false;
     bool preprocess();
 };

@@ -77,12 +77,32 @@ def spmm_csr_f32(indptr, indices, values, X):
     return Y
 
 
-def spmm_csr_f64(indptr, indices, values, X):
+def spmm_csr_f64(indptr, indices, values, X, threads: int = 1):
+    """R = A X and S = |A| |X| in fp64.  ``threads`` > 1 runs the same C routine on
+    consecutive row ranges from that many host threads (ctypes releases the GIL)."""
     ip, ix, v, X = _i32(indptr), _i32(indices), _f32(values), _f32(X)
-    R = np.empty((ip.size - 1, X.shape[1]), dtype=np.float64)
+    n, N = ip.size - 1, X.shape[1]
+    R = np.empty((n, N), dtype=np.float64)
     S = np.empty_like(R)
-    lib().oracle_spmm_csr_f64(_p(ip, C.c_int32), _p(ix, C.c_int32), _p(v, C.c_float), ip.size - 1,
-                              _p(X, C.c_float), _p(R, C.c_double), _p(S, C.c_double), X.shape[1])
+    fn = lib().oracle_spmm_csr_f64
+
+    def rows(r0, r1):          # indptr entries stay absolute offsets into idx / val
+        fn(_p(ip[r0:], C.c_int32), _p(ix, C.c_int32), _p(v, C.c_float), r1 - r0, _p(X, C.c_float),
+           _p(R[r0:], C.c_double), _p(S[r0:], C.c_double), N)
+
+    if threads <= 1 or n < 2 * threads:
+        rows(0, n)
+        return R, S
+    import threading
+    # ranges of about equal non-zeros
+    cuts = np.searchsorted(ip, np.linspace(int(ip[0]), int(ip[-1]), threads + 1)[1:-1]).tolist()
+    bounds = [0] + [min(max(int(c), 0), n) for c in cuts] + [n]
+    ts = [threading.Thread(target=rows, args=(bounds[i], bounds[i + 1])) for i in range(threads)
+          if bounds[i + 1] > bounds[i]]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
     return R, S
 
 

@@ -41,6 +41,17 @@ def test_cli_without_gpu_says_so(pkg):
 
 
 @pytest.mark.gpu
+def test_operator_error_paths(gpu):
+    """bin/operator_check: a refused launch is reported by do_test and nothing more is
+    launched, the operator computes again afterwards, a host pointer is refused."""
+    exe = EXE.parent / "operator_check"
+    assert exe.exists(), "operator_check was not built"
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("ok:") == 4 and "FAIL" not in r.stdout
+
+
+@pytest.mark.gpu
 def test_cli_check_and_timing(gpu, tmp_path):
     graphs, meta = write_graph(tmp_path, "mix", seed=11)
     r = subprocess.run([str(EXE), "--graphs", str(graphs), "--meta", str(meta), "mix", "60"],
@@ -75,3 +86,22 @@ def test_cli_sweep_mode(gpu, tmp_path):
     assert len(lines) == 2 * 113
     assert {(l[0], l[1]) for l in lines} == {("1", "a"), ("2", "b")}
     assert [int(l[2]) for l in lines[:113]] == list(range(16, 129))
+
+
+@pytest.mark.gpu
+def test_cli_saved_state_is_loaded_by_the_next_run(gpu, tmp_path):
+    graphs, meta = write_graph(tmp_path, "mix", seed=13)
+    cmd = [str(EXE), "--graphs", str(graphs), "--meta", str(meta), "--save-state", "mix", "48"]
+    first = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+    assert first.returncode == 0, first.stdout + first.stderr
+    assert (meta / "mix.accelstate").exists() and "loaded from saved state" not in first.stderr
+    second = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+    assert second.returncode == 0, second.stdout + second.stderr
+    assert "loaded from saved state" in second.stderr and "validation pass!" in second.stdout
+    # a state that belongs to another graph is a stale cache entry: recomputed, not an error
+    graphs2, meta2 = write_graph(tmp_path, "other", seed=14)
+    (meta / "mix.accelstate").rename(meta2 / "other.accelstate")
+    third = subprocess.run([str(EXE), "--graphs", str(graphs2), "--meta", str(meta2), "other", "48"],
+                           capture_output=True, text=True, timeout=120)
+    assert third.returncode == 0, third.stdout + third.stderr
+    assert "loaded from saved state" not in third.stderr and "validation pass!" in third.stdout

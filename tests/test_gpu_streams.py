@@ -117,6 +117,106 @@ def test_graph_capture_and_replay(gpu, hip):
     dX.close(); dY.close(); op.close()
 
 
+def test_second_stream_is_refused_while_the_first_run_is_in_flight(gpu, hip):
+    """The partial-sum buffer of a handle is shared by its runs: a run on another stream
+    while the previous one has not finished is an error, not silent corruption."""
+    g = gpu.synthetic.cfg2()
+    N = 128
+    X = gpu.synthetic.dense_operand("cfg2", g.n_cols, N)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    assert op.info.n_split_rows > 0
+    dX, dY = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer(g.n_rows * N * 4)
+    s1, s2 = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(s1)))
+    ok(hip.hipStreamCreate(C.byref(s2)))
+    op.run(dX, dY, N, stream=s1.value)
+    ok(hip.hipStreamSynchronize(s1))
+    op.run(dX, dY, N, stream=s2.value)                    # the first run has finished: fine
+    ok(hip.hipStreamSynchronize(s2))
+    for _ in range(300):                                  # some 40 ms of queued work on s1
+        op.run(dX, dY, N, stream=s1.value)
+    with pytest.raises(gpu.AccelError) as e:
+        op.run(dX, dY, N, stream=s2.value)
+    assert e.value.status == gpu._lib.ERR_STATE and "another stream" in e.value.message
+    op.run(dX, dY, N, stream=s1.value)                    # the same stream is always fine
+    ok(hip.hipStreamSynchronize(s1))
+    op.run(dX, dY, N, stream=s2.value)                    # and so is the other one, after the wait
+    ok(hip.hipStreamSynchronize(s2))
+    Y = dY.to_numpy(np.float32, (g.n_rows, N))
+    assert so.check(Y, g.indptr, g.indices, g.values, X) <= so.TOL
+    ok(hip.hipStreamDestroy(s1))
+    ok(hip.hipStreamDestroy(s2))
+    dX.close(); dY.close(); op.close()
+
+
+def test_reserve_before_capture(gpu, hip):
+    """A captured run must not grow the partial-sum buffer: without accel_reserve a first
+    run with a larger N inside a capture is refused; with it, the graph replays and later
+    eager runs with smaller N leave the graph valid."""
+    g, X, op = make_case(gpu, 34, 96)
+    N = 96
+    dX, dY = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer(g.n_rows * N * 4)
+    X16 = np.ascontiguousarray(X[:, :16])
+    dX16, dY16 = gpu.DeviceBuffer.from_numpy(X16), gpu.DeviceBuffer(g.n_rows * 16 * 4)
+    op.run(dX16, dY16, 16)                                # the buffer now fits N = 16 only
+    op.synchronize()
+    s = C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(s)))
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamBeginCapture(s, 0))
+    with pytest.raises(gpu.AccelError) as e:
+        op.run(dX, dY, N, stream=s.value)
+    assert e.value.status == gpu._lib.ERR_STATE and "accel_reserve" in e.value.message
+    hip.hipStreamEndCapture(s, C.byref(graph))            # nothing was recorded; end the capture
+    if graph.value:
+        hip.hipGraphDestroy(graph)
+    op.reserve(N)
+    graph = C.c_void_p()
+    ok(hip.hipStreamBeginCapture(s, 0))
+    op.run(dX, dY, N, stream=s.value)
+    ok(hip.hipStreamEndCapture(s, C.byref(graph)))
+    ok(hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0))
+    for rep in range(3):
+        dY.fill_u32(0x7FC00000)
+        op.run(dX16, dY16, 16)                            # eager runs with a smaller N in between
+        op.synchronize()
+        ok(hip.hipGraphLaunch(gexec, s))
+        ok(hip.hipStreamSynchronize(s))
+        Y = dY.to_numpy(np.float32, (g.n_rows, N))
+        assert so.check(Y, g.indptr, g.indices, g.values, X) <= so.TOL, f"replay {rep}"
+    ok(hip.hipGraphExecDestroy(gexec))
+    ok(hip.hipGraphDestroy(graph))
+    ok(hip.hipStreamDestroy(s))
+    for b in (dX, dY, dX16, dY16):
+        b.close()
+    op.close()
+
+
+def test_operands_the_gpu_cannot_use_are_refused(gpu):
+    """A host address or an allocation that is too small comes back as ACCEL_ERR_ARG from the
+    C ABI (given as raw addresses, so that the host-side checks of the binding do not see them)."""
+    g, X, op = make_case(gpu, 35, 32)
+    N = 32
+    dX, dY = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer(g.n_rows * N * 4)
+    host_y = np.zeros((g.n_rows, N), np.float32)
+    small = gpu.DeviceBuffer(g.n_rows * N * 4 - 64)
+    for args in ((X.ctypes.data, dY.address), (dX.address, host_y.ctypes.data), (dX.address, small.address),
+                 (dX.address + 64, dY.address)):
+        with pytest.raises(gpu.AccelError) as e:
+            op.run(args[0], args[1], N)
+        assert e.value.status == gpu._lib.ERR_ARG, e.value
+    with pytest.raises(gpu.AccelError):                   # the binding's own check
+        op.run(X, dY, N)
+    with pytest.raises(gpu.AccelError):
+        op.run(dX, small, N)
+    op.run(dX, dY, N)                                     # good operands still run
+    op.synchronize()
+    assert so.check(dY.to_numpy(np.float32, (g.n_rows, N)), g.indptr, g.indices, g.values, X) <= so.TOL
+    for b in (dX, dY, small):
+        b.close()
+    op.close()
+
+
 def test_torch_tensors_as_operands(gpu):
     """torch tensors (data_ptr, torch's current stream) straight into the C ABI, in a
     process that imports torch first so that one HIP runtime serves both."""

@@ -148,3 +148,30 @@ def test_product_does_not_import_the_oracle():
         if f.is_file():
             text = f.read_text(errors="ignore")
             assert "oracle" not in text.lower(), f"{f} mentions the oracle"
+
+
+def test_binding_refuses_host_arrays_as_dense_operands(pkg):
+    """run/run_epilogue/time take device memory; a numpy array (a host address) or an
+    object that says it is too small is refused before anything reaches the library."""
+    L = pkg._lib
+    with pytest.raises(pkg.AccelError) as e:
+        L.dev_ptr(np.zeros(8, np.float32), 32, "X")
+    assert e.value.status == L.ERR_ARG and "host" in e.value.message
+
+    class FakeTensor:
+        def __init__(self, n, cuda):
+            self.n, self.is_cuda = n, cuda
+        def data_ptr(self):
+            return 0x1000
+        def numel(self):
+            return self.n
+        def element_size(self):
+            return 4
+
+    with pytest.raises(pkg.AccelError):
+        L.dev_ptr(FakeTensor(8, False), 32, "X")          # a CPU tensor
+    with pytest.raises(pkg.AccelError):
+        L.dev_ptr(FakeTensor(7, True), 32, "Y")           # too small
+    assert L.dev_ptr(FakeTensor(8, True), 32, "Y").value == 0x1000
+    assert L.dev_ptr(None, 4, "bias") is None
+    assert L.dev_ptr(0x2000, 1 << 40, "X").value == 0x2000  # raw addresses are the library's to check

@@ -79,3 +79,15 @@ def test_scaled_error_catches_a_dropped_term():
     v[7] = 0.0
     assert so.scaled_error(so.spmm_scipy32(g.indptr, g.indices, v, X), R, S) > 100 * so.TOL
     assert so.scaled_error(so.spmm_scipy32(g.indptr, g.indices, g.values, X), R, S) <= so.TOL
+
+
+def test_threaded_fp64_oracle_is_the_same_routine_on_row_ranges():
+    import helpers
+    from oracle import c_oracle
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=1, n_long=20), seed=1)
+    X = np.random.default_rng(0).standard_normal((g.n_cols, 20)).astype(np.float32)
+    R1, S1 = c_oracle.spmm_csr_f64(g.indptr, g.indices, g.values, X)
+    R2, S2 = c_oracle.spmm_csr_f64(g.indptr, g.indices, g.values, X, threads=5)
+    assert np.array_equal(R1, R2) and np.array_equal(S1, S2)
+    R3, S3 = c_oracle.spmm_csr_f64(g.indptr[50:201], g.indices, g.values, X, threads=3)   # a slab of rows
+    assert np.array_equal(R3, R1[50:200]) and np.array_equal(S3, S1[50:200])
