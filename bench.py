@@ -23,22 +23,46 @@ import numpy as np
 HBM_PEAK_GBS = 8000.0
 
 
+KERNEL_SOURCES = ("spmm.hip", "preprocess.hip", "internal.h")
+
+
+def kernel_source_hash():
+    """First 16 hex digits of the SHA-256 over the sources that decide what the gather kernel
+    does and in which order (kernels, launch plan, shared constants)."""
+    import hashlib
+    h = hashlib.sha256()
+    base = os.path.join(os.path.dirname(os.path.abspath(__file__)), "iccad-accel-gcn_amd", "csrc")
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(base, name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def recorded_traffic(workload, N):
-    """HBM bytes per launch from the committed rocprofv3 counter runs, if this
-    workload was profiled (the counters cannot be read from inside a timing run)."""
+    """HBM bytes per launch from the committed rocprofv3 counter runs (the counters cannot be
+    read from inside a timing run).  Every entry records the hash of the kernel sources it was
+    taken with: an entry taken with other sources is reported as stale, not as this run's."""
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "spmm_gather_traffic.json")
     try:
         with open(path) as f:
-            return json.load(f).get(f"{workload}/N{N}", {}).get("traffic_bytes")
+            entry = json.load(f).get(f"{workload}/N{N}")
     except OSError:
-        return None
+        return None, "no profile file"
+    if not entry:
+        return None, "this workload was not profiled"
+    now = kernel_source_hash()
+    if entry.get("source_sha16") != now:
+        return None, (f"profiles/spmm_gather_traffic.json holds {entry.get('traffic_bytes')} bytes for this "
+                      f"workload, taken with kernel sources {entry.get('source_sha16', 'of unknown hash')}; "
+                      f"the sources now hash to {now}")
+    return entry.get("traffic_bytes"), None
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def cpu_baseline(g, X, N, budget_s=15.0):
+def cpu_baseline(g, X, N, budget_s=10.0):
     """scipy csr @ X (fp32, one thread) on the first rows of the CSR that fit the
     time budget; the checker only, never the measured path."""
     from oracle import spmm_oracle as so
@@ -66,46 +90,29 @@ def cpu_baseline(g, X, N, budget_s=15.0):
                       f"({nz} of {g.nnz} non-zeros), N={N}, 1 thread"}, n_rows, Y
 
 
-def fixture_graph(pkg, name, seed=0, sigma=0):
-    """A graph with exactly the degree sequence of one of the reference's
-    benchmark graphs (recovered from its golden .block4 metadata: degree, first
-    row and row count of every block; rows no block covers have degree 0), rows
-    in shuffled order, values GCN-normalised.  The real edge lists are not
-    available offline, so the columns are synthetic: uniform random (sigma = 0),
-    or, to model a vertex order with locality, row id + N(0, sigma) (duplicates
-    inside a row merge, so such a graph has slightly fewer non-zeros)."""
-    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "golden"))
-    import block4_codec
-    b = block4_codec.load(name).astype(np.int64)
-    is_long = b[:, 0] > 384
-    first = np.ones(len(b), dtype=bool)
-    first[1:] = ~(is_long[1:] & (b[1:, 1] == b[:-1, 1]))
-    b = b[first]
-    n_rows_blk = np.where(b[:, 0] > 384, 1, b[:, 3] & 0xFFFF)
-    n = int((b[:, 1] + n_rows_blk).max())
-    deg = np.zeros(n, dtype=np.int64)
-    deg[np.repeat(b[:, 1], n_rows_blk) + (np.arange(n_rows_blk.sum()) - np.repeat(np.cumsum(n_rows_blk) - n_rows_blk, n_rows_blk))] = np.repeat(b[:, 0], n_rows_blk)
-    rng = np.random.default_rng(seed)
-    deg = rng.permutation(deg)
-    src = np.repeat(np.arange(n, dtype=np.int64), deg)
-    if sigma > 0:
-        dst = np.clip(src + np.rint(rng.standard_normal(src.size) * sigma).astype(np.int64), 0, n - 1)
-    else:
-        dst = rng.integers(0, n, size=src.size, dtype=np.int64)
-    syn = pkg.synthetic
-    indptr, indices = syn._csr_from_edges(src, dst, n, n)
-    g = syn.Graph(name, indptr, indices, syn._gcn_values(indptr, indices), n, n)
-    return g
-
-
-def uniform_graph(pkg, n_rows, degree, n_cols, seed=0):
-    """Every row has `degree` non-zeros with columns uniform over n_cols (repeats
-    allowed): a probe of the gather rate for an X of a chosen size."""
-    rng = np.random.default_rng(seed)
-    indptr = (np.arange(n_rows + 1, dtype=np.int64) * degree).astype(np.int32)
-    indices = rng.integers(0, n_cols, size=n_rows * degree).astype(np.int32)
-    values = rng.random(n_rows * degree, dtype=np.float32)
-    return pkg.synthetic.Graph(f"uniform:{n_rows}:{degree}:{n_cols}", indptr, indices, values, n_rows, n_cols)
+def load_workload(syn, spec, cache_dir):
+    """The workload's CSR, generated once per machine: the arrays are kept under
+    ``cache_dir`` so that repeated runs (profiler passes) skip the generator."""
+    import hashlib
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "iccad-accel-gcn_amd", "synthetic.py"), "rb") as f:
+        tag = hashlib.sha256(f.read() + spec.encode()).hexdigest()[:16]
+    path = os.path.join(cache_dir, f"{spec.replace(':', '-')}-{tag}.npz") if cache_dir else None
+    if path and os.path.exists(path):
+        try:
+            z = np.load(path)
+            return syn.Graph(spec, z["indptr"], z["indices"], z["values"], int(z["n_rows"]), int(z["n_cols"])), True
+        except Exception:
+            pass                                           # unreadable cache entry: generate again
+    g = syn.workload(spec)
+    if path:
+        try:
+            os.makedirs(cache_dir, exist_ok=True)
+            tmp = path + f".{os.getpid()}.tmp.npz"
+            np.savez(tmp, indptr=g.indptr, indices=g.indices, values=g.values, n_rows=g.n_rows, n_cols=g.n_cols)
+            os.replace(tmp, path)
+        except OSError:
+            pass
+    return g, False
 
 
 def rocsparse_baseline(pkg, op, g, dX, N, iters=10):
@@ -190,6 +197,8 @@ def main():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run the plain copy kernel over this many MiB, --steps times "
                          "(known-size reference for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--cache-dir", default="/tmp/accelgcn_bench_cache",
+                    help="where generated workloads are kept between runs ('' = do not keep them)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures one GPU only (the path has no multi-GPU part); "
@@ -232,20 +241,13 @@ def main():
     N = a.N or syn.WORKLOAD_N.get(a.workload, (64,))[0]
 
     t0 = time.time()
-    if a.workload.startswith("fixture:"):
-        g = fixture_graph(pkg, a.workload.split(":", 1)[1])
-    elif a.workload.startswith("uniform:"):             # uniform:<rows>:<degree>:<cols>
-        _, n_rows, degree, n_cols = a.workload.split(":")
-        g = uniform_graph(pkg, int(n_rows), int(degree), int(n_cols))
-    elif a.workload.startswith("local:"):               # local:<name>:<sigma>
-        _, name, sigma = a.workload.split(":")
-        g = fixture_graph(pkg, name, sigma=int(sigma))
-    elif a.workload in syn.WORKLOADS:
-        g = syn.WORKLOADS[a.workload]()
-    else:
-        sys.exit(f"bench.py: unknown workload {a.workload}")
+    try:
+        g, cached = load_workload(syn, a.workload, a.cache_dir)
+    except (ValueError, KeyError) as e:
+        sys.exit(f"bench.py: {e}")
     X = syn.dense_operand(a.workload, g.n_cols, N)
-    log(f"[bench] {a.workload}: rows={g.n_rows} nnz={g.nnz} N={N} generated in {time.time() - t0:.1f}s")
+    log(f"[bench] {a.workload}: rows={g.n_rows} nnz={g.nnz} N={N} "
+        f"{'loaded from the cache' if cached else 'generated'} in {time.time() - t0:.1f}s")
 
     t0 = time.time()
     op = pkg.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols)
@@ -257,6 +259,19 @@ def main():
     log(f"[bench] upload {t_upload * 1e3:.0f} ms, preprocess {info.preprocess_ms:.1f} ms: "
         f"blocks={info.n_blocks} long_rows={info.n_long_rows} long_blocks={info.n_long_blocks} "
         f"zero_rows={info.n_zero_rows} max_degree={info.max_degree}")
+    # the same products from a saved state instead (accel_save_state / accel_load_state)
+    import tempfile
+    from_cache_ms = None
+    with tempfile.TemporaryDirectory() as td:
+        state = os.path.join(td, "bench.accelstate")
+        op.save_state(state)
+        state_mb = os.path.getsize(state) / 1e6
+        op2 = pkg.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols)
+        op2.load_state(state)
+        op2.load_state(state)                        # second load: file in the page cache, kernels loaded
+        from_cache_ms = op2.info.preprocess_ms
+        op2.close()
+    log(f"[bench] preprocess from a saved state ({state_mb:.1f} MB): {from_cache_ms:.1f} ms")
     dX = pkg.DeviceBuffer.from_numpy(X)
     dY = pkg.DeviceBuffer(g.n_rows * N * 4)
     dY.fill_u32(0x7FC00000)
@@ -288,6 +303,8 @@ def main():
     alg_bytes = g.nnz * 8 + g.n_cols * N * 4 + g.n_rows * N * 4
     main_avg_ms = float(np.mean(main_ms))
     achieved = alg_bytes / (main_avg_ms * 1e-3) / 1e9
+    achieved_all = alg_bytes / (float(np.mean(tot_ms)) * 1e-3) / 1e9
+    traffic, traffic_note = recorded_traffic(a.workload, N)
     result = {
         "metric": "SpMM GFLOP/s (2*nnz*N), fp32",
         "value": round(flops / (ms_per_step * 1e-3) / 1e9, 2),
@@ -300,16 +317,20 @@ def main():
                    "rows": g.n_rows, "nnz": g.nnz, "N": N, "blocks": int(info.n_blocks),
                    "preprocess_ms": round(info.preprocess_ms, 2),
                    "preprocess_first_call_ms": round(first_preprocess_ms, 2),
+                   "preprocess_from_cache_ms": round(from_cache_ms, 2),
                    "reference_protocol_ms": round(ref_protocol_ms, 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": recorded_traffic(a.workload, N),
+                     "traffic": traffic,
                      "kernel": "spmm_gather_kernel", "kernel_ms_avg": round(main_avg_ms, 5),
                      "kernel_ms_min": round(float(np.min(main_ms)), 5),
                      "all_kernels_ms_avg": round(float(np.mean(tot_ms)), 5),
                      "all_kernels_ms_median": round(float(np.median(tot_ms)), 5),
-                     "algorithmic_bytes": alg_bytes},
+                     "frac_all_kernels": round(achieved_all / HBM_PEAK_GBS, 4),
+                     "algorithmic_bytes": alg_bytes, "kernel_source_sha16": kernel_source_hash()},
     }
+    if traffic_note:
+        result["roofline"]["traffic_stale"] = traffic_note
 
     if a.compare_rocsparse:
         rs, Yr = rocsparse_baseline(pkg, op, g, dX, N)

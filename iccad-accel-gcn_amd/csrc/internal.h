@@ -15,10 +15,7 @@ constexpr int kDegBound = ACCEL_DEG_BOUND;            // non-zeros per block4 en
 constexpr int kSlices = ACCEL_SLICES_PER_BLOCK;       // slices per entry (metadata ABI)
 constexpr int kSliceNz = kDegBound / kSlices;         // 32
 constexpr int kXcds = 8;                              // accelerator dies, each with its own L2
-#ifndef ACCEL_WAVES_PER_GROUP
-#define ACCEL_WAVES_PER_GROUP 4
-#endif
-constexpr int kWavesPerGroup = ACCEL_WAVES_PER_GROUP; // wavefronts (work units) per workgroup
+constexpr int kWavesPerGroup = 4;                     // wavefronts (work units) per workgroup (1, 2, 8: within 2 %)
 
 constexpr int kMaxGroups = 64;                        // column groups of the launch plan (8..64)
 
@@ -30,17 +27,15 @@ constexpr int kMaxGroups = 64;                        // column groups of the la
 __host__ __device__ inline int col_group(int c, int groups) { return (c >> 3) & (groups - 1); }
 
 // Column groups a split row of degree d is stored in: as many as leave a group about
-// ACCEL_GROUP_MIN_PIECE non-zeros, 8 at least, 64 at most (a power of two); `forced`
+// kGroupMinPiece non-zeros, 8 at least, 64 at most (a power of two); `forced`
 // (8..64) overrides the rule.  Short split rows keep few, long pieces; very long rows
 // are spread over many groups, whose share of X is small enough to stay in one L2.
-#ifndef ACCEL_GROUP_MIN_PIECE
-#define ACCEL_GROUP_MIN_PIECE 96
-#endif
+constexpr int kGroupMinPiece = 96;                    // 48 and 192 measured: each better on one workload, worse on another
 __host__ __device__ inline int row_groups(int d, int forced)
 {
     if (forced) return forced;
     int g = kXcds;
-    while (g < kMaxGroups && d / (2 * g) >= ACCEL_GROUP_MIN_PIECE) g *= 2;
+    while (g < kMaxGroups && d / (2 * g) >= kGroupMinPiece) g *= 2;
     return g;
 }
 // Pieces are binned by (groups of their row, group): 8 + 16 + 32 + 64 bins.
@@ -112,6 +107,7 @@ struct accel_handle {
     bool local = false;               // most non-zeros lie near the diagonal (sampled)
     int64_t n_split_rows = 0;         // rows with more than plan_split non-zeros
     int64_t n_big_rows = 0;           // of those, rows with more than 32 * plan_split
+    int64_t n_wide_rows = 0;          // rows with more than 1,024 non-zeros (regrouped by a workgroup each)
     int64_t n_blocks = 0, n_long_blocks = 0, n_long_rows = 0, n_zero_rows = 0;
     int32_t max_degree = 0;
     double preprocess_ms = 0.0;

@@ -154,9 +154,14 @@ struct Stats {
     int n_split_rows;   // rows with more non-zeros than the plan's split threshold
     int n_big_rows;     // rows with more than 32 times that
     int n_split_rows_alt, n_big_rows_alt;   // the same two for the alternative threshold
+    int n_wide_rows;    // rows with more than kGroupWaveMax non-zeros
     int sampled_nz;     // non-zeros looked at by locality_kernel
     int local_nz;       // ... whose column lies near their row
 };
+
+// Split rows of up to this many non-zeros are regrouped by one wavefront each, longer ones
+// by a workgroup each (group_long_rows_*).
+constexpr int kGroupWaveMax = 1024;
 
 __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restrict__ indptr,
                                                           int64_t rows, int64_t nnz,
@@ -165,8 +170,9 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
                                                           int alt_split_deg)
 {
     // grid-stride over rows; one set of atomics per workgroup
-    __shared__ int part[kThreads / 64][10];
+    __shared__ int part[kThreads / 64][11];
     int bad = 0, unsorted = 0, dmax = 0, zero = 0, lrow = 0, lblk = 0, srow = 0, brow = 0, srow2 = 0, brow2 = 0;
+    int wrow = 0;
     for (int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x; r < rows;
          r += (int64_t)gridDim.x * kThreads) {
         const int a = indptr[r], b = indptr[r + 1];
@@ -185,6 +191,7 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
         brow += d > 32 * split_deg;
         srow2 += d > alt_split_deg;
         brow2 += d > 32 * alt_split_deg;
+        wrow += d > kGroupWaveMax;
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -198,19 +205,20 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
         brow += __shfl_xor(brow, off);
         srow2 += __shfl_xor(srow2, off);
         brow2 += __shfl_xor(brow2, off);
+        wrow += __shfl_xor(wrow, off);
     }
     const int w = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) {
         part[w][0] = bad; part[w][1] = unsorted; part[w][2] = dmax;
         part[w][3] = zero; part[w][4] = lrow; part[w][5] = lblk; part[w][6] = srow; part[w][7] = brow;
-        part[w][8] = srow2; part[w][9] = brow2;
+        part[w][8] = srow2; part[w][9] = brow2; part[w][10] = wrow;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int q = 1; q < kThreads / 64; q++) {
             bad |= part[q][0]; unsorted |= part[q][1]; dmax = max(dmax, part[q][2]);
             zero += part[q][3]; lrow += part[q][4]; lblk += part[q][5]; srow += part[q][6]; brow += part[q][7];
-            srow2 += part[q][8]; brow2 += part[q][9];
+            srow2 += part[q][8]; brow2 += part[q][9]; wrow += part[q][10];
         }
         if (bad) atomicOr(&st->bad_indptr, 1);
         if (unsorted) atomicOr(&st->unsorted, 1);
@@ -222,22 +230,26 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
         if (brow) atomicAdd(&st->n_big_rows, brow);
         if (srow2) atomicAdd(&st->n_split_rows_alt, srow2);
         if (brow2) atomicAdd(&st->n_big_rows_alt, brow2);
+        if (wrow) atomicAdd(&st->n_wide_rows, wrow);
     }
 }
 
 // Does the matrix have its non-zeros near the diagonal (of the rows x cols rectangle)?
 // Every kLocalityStride-th row contributes up to kLocalitySample of its non-zeros, evenly spaced; one counts
-// as local when its column is within `band` columns of the row's place.  Runs after indptr
-// has been validated.
+// as local when its column is within `band` columns of the row's place.  Rows whose indptr
+// entries point outside [0, nnz) are skipped (degree_kernel reports them).
 constexpr int kLocalityStride = 16, kLocalitySample = 16;
 __global__ __launch_bounds__(kThreads) void locality_kernel(const int32_t *__restrict__ indptr,
                                                             const int32_t *__restrict__ idx, int64_t rows,
-                                                            int64_t cols, int band, Stats *__restrict__ st)
+                                                            int64_t cols, int64_t nnz, int band,
+                                                            Stats *__restrict__ st)
 {
     const int64_t r = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * kLocalityStride;
     int seen = 0, local = 0;
     if (r < rows) {
-        const int a = indptr[r], d = indptr[r + 1] - a, n = min(d, kLocalitySample);
+        int a = indptr[r], d = indptr[r + 1] - a;
+        if (a < 0 || d < 0 || (int64_t)a + d > nnz) d = 0;     // invalid indptr: reported by degree_kernel
+        const int n = min(d, kLocalitySample);
         const int64_t place = rows > 1 ? r * (cols - 1) / (rows - 1) : 0;
         for (int i = 0; i < n; i++) {                    // spread over the row, whatever its order
             const int64_t off = (int64_t)idx[a + (int)((int64_t)i * d / n)] - place;
@@ -260,12 +272,20 @@ __global__ __launch_bounds__(kThreads) void index_check_kernel(const int32_t *__
                                                                int64_t nnz, int64_t cols,
                                                                Stats *__restrict__ st)
 {
+    // 16-byte loads over the aligned middle of the array, single words at its two ends
     int bad = 0;
-    for (int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x; p < nnz;
-         p += (int64_t)gridDim.x * kThreads) {
-        const int c = idx[p];
-        bad |= (c < 0) | ((int64_t)c >= cols);
+    auto look = [&](int c) { bad |= (c < 0) | ((int64_t)c >= cols); };
+    const int64_t tid = (int64_t)blockIdx.x * kThreads + threadIdx.x, step = (int64_t)gridDim.x * kThreads;
+    int64_t head = (int64_t)((16 - (reinterpret_cast<uintptr_t>(idx) & 15)) & 15) / 4;
+    if (head > nnz) head = nnz;
+    const int64_t n4 = (nnz - head) / 4;
+    const int4 *v = reinterpret_cast<const int4 *>(idx + head);
+    for (int64_t i = tid; i < n4; i += step) {
+        const int4 c = v[i];
+        look(c.x); look(c.y); look(c.z); look(c.w);
     }
+    for (int64_t p = tid; p < head; p += step) look(idx[p]);
+    for (int64_t p = head + 4 * n4 + tid; p < nnz; p += step) look(idx[p]);
     if (__ballot(bad) && (threadIdx.x & 63) == 0) atomicOr(&st->bad_index, 1);
 }
 
@@ -402,6 +422,10 @@ struct DevBuf {  // frees on scope exit; with an arena, the arena owns the memor
 };
 
 inline unsigned grid_for(int64_t n) { return (unsigned)((n + kThreads - 1) / kThreads); }
+// Workgroups of degree_kernel: each ends with a dozen atomics on the same few words, which
+// the memory system applies one after the other (2,048 workgroups: 160 us on 2.45 M rows,
+// almost all of it those atomics).
+constexpr unsigned kDegreeGroups = 256;
 
 // Sorts n (key, position) pairs by key, stably, in as many 8-bit passes as max_key needs.
 // keys is used as one of the two key buffers; *sorted_keys / *sorted_vals point at the
@@ -569,6 +593,86 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
     }
 }
 
+// The same regrouping with one wavefront per row, four rows per workgroup: for the many
+// split rows of a few hundred non-zeros a workgroup per row is mostly barriers and idle
+// lanes, and four times as many rows are in flight this way.  No workgroup barrier: a
+// wavefront only touches its own part of LDS, whose accesses execute in program order.
+__global__ __launch_bounds__(kThreads) void group_long_rows_wave_kernel(
+    const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
+    const float *__restrict__ val, const int32_t *__restrict__ perm,
+    const int32_t *__restrict__ s_indptr, int64_t first_long_row, int n_rows, int forced_groups,
+    int32_t *__restrict__ s_idx, float *__restrict__ s_val, int *__restrict__ counts)
+{
+    static_assert(kMaxGroups == 64, "one lane per column group");
+    __shared__ int cnt[kThreads / 64][kMaxGroups];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lr = (int)blockIdx.x * (kThreads / 64) + w;
+    if (lr >= n_rows) return;                            // the whole wavefront leaves
+    const int64_t r = first_long_row + lr;
+    const int64_t src0 = indptr[perm ? perm[r] : r];
+    const int64_t dst0 = s_indptr[r];
+    const int d = s_indptr[r + 1] - s_indptr[r];
+    const int ng = row_groups(d, forced_groups);
+    int *my = cnt[w];
+    my[lane] = 0;
+    __builtin_amdgcn_wave_barrier();
+    for (int i = lane; i < d; i += 64) atomicAdd(&my[col_group(idx[src0 + i], ng)], 1);
+    __builtin_amdgcn_wave_barrier();
+    const int c = my[lane];                              // lane g holds the size of group g
+    if (counts) counts[(int64_t)lr * kMaxGroups + lane] = c;
+    int inc = c;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int t = __shfl_up(inc, off);
+        if (lane >= off) inc += t;
+    }
+    __builtin_amdgcn_wave_barrier();
+    my[lane] = inc - c;                                  // where group g starts; moves on as it fills
+    __builtin_amdgcn_wave_barrier();
+    for (int c0 = 0; c0 < d; c0 += 64) {
+        const int i = c0 + lane;
+        const bool valid = i < d;
+        const int col = valid ? idx[src0 + i] : 0;
+        const float v = valid ? val[src0 + i] : 0.0f;
+        const int g = col_group(col, ng);
+        unsigned long long peers = __ballot(valid);      // lanes with the same group
+#pragma unroll
+        for (int b = 0; b < 6; b++) {
+            const bool bit = (g >> b) & 1;
+            const unsigned long long bal = __ballot(bit);
+            peers &= bit ? bal : ~bal;
+        }
+        const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+        int pos = 0;
+        if (valid) pos = my[g] + rank;
+        __builtin_amdgcn_wave_barrier();
+        if (valid) {
+            s_idx[dst0 + pos] = col;
+            s_val[dst0 + pos] = v;
+            if (rank == 0) my[g] += __popcll(peers);     // one lane per group present
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// Regroups the n_long split rows (the last rows of the sorted order, ascending by
+// length, n_wide of them longer than kGroupWaveMax).
+static void launch_group_long_rows(const int32_t *indptr, const int32_t *idx, const float *val,
+                                   const int32_t *perm, const int32_t *s_indptr, int64_t first_long,
+                                   int64_t n_long, int64_t n_wide, int forced_groups, int32_t *s_idx,
+                                   float *s_val, int *counts, hipStream_t s)
+{
+    const int64_t n_narrow = n_long - n_wide;
+    if (n_narrow > 0)
+        group_long_rows_wave_kernel<<<dim3((unsigned)((n_narrow + kThreads / 64 - 1) / (kThreads / 64))),
+                                      dim3(kThreads), 0, s>>>(
+            indptr, idx, val, perm, s_indptr, first_long, (int)n_narrow, forced_groups, s_idx, s_val, counts);
+    if (n_wide > 0)
+        group_long_rows_kernel<<<dim3((unsigned)n_wide), dim3(kThreads), 0, s>>>(
+            indptr, idx, val, perm, s_indptr, first_long + n_narrow, forced_groups, s_idx, s_val,
+            counts ? counts + n_narrow * kMaxGroups : nullptr);
+}
+
 // ---------------------------------------------------------------------------
 // Partition
 // ---------------------------------------------------------------------------
@@ -645,9 +749,7 @@ __device__ __forceinline__ int64_t plan_index(int queue, int pos)
 // Rows stored in up to this many column groups follow the caller's row ids inside their
 // bins; the longer ones keep "largest first" (they touch all of X whatever their id, and the
 // hub workload measured 2 % faster that way: 2.31 against 2.36 ms at N = 256).
-#ifndef ACCEL_ID_ORDER_MAX_GROUPS
-#define ACCEL_ID_ORDER_MAX_GROUPS 8
-#endif
+constexpr int kIdOrderMaxGroups = 8;
 __global__ __launch_bounds__(kThreads) void long_row_key_kernel(const uint32_t *__restrict__ perm,
                                                                 const int32_t *__restrict__ s_indptr,
                                                                 int forced_groups, int key_shift,
@@ -658,7 +760,7 @@ __global__ __launch_bounds__(kThreads) void long_row_key_kernel(const uint32_t *
     if (lr >= n_long) return;
     const int64_t row = first_long + lr;
     const int ng = row_groups(s_indptr[row + 1] - s_indptr[row], forced_groups);
-    if (ng <= ACCEL_ID_ORDER_MAX_GROUPS)
+    if (ng <= kIdOrderMaxGroups)
         key[lr] = (perm ? perm[row] : (uint32_t)row) >> key_shift;
     else
         key[lr] = (uint32_t)(n_long - 1 - lr) >> key_shift;   // largest rows first
@@ -829,9 +931,7 @@ __global__ __launch_bounds__(kThreads) void queue_first_kernel(const int *__rest
 // long chain.  They are the light units with the highest ids of the queue's share, i.e.
 // they lie in the band of rows the die is working on at that time anyway.
 // heavy_before[s] = heavy units among the first s, [n] = all.
-#ifndef ACCEL_TAIL_LIGHT
-#define ACCEL_TAIL_LIGHT 2048                // two rounds of the 1,024 wavefronts a die holds
-#endif
+constexpr int kTailLight = 2048;             // two rounds of the 1,024 wavefronts a die holds
 __global__ __launch_bounds__(kThreads) void place_short_units_kernel(
     const int4 *__restrict__ units, const uint32_t *__restrict__ order, const int *__restrict__ running,
     const int *__restrict__ heavy_before, int n, QueueCuts qc, const int *__restrict__ first,
@@ -845,7 +945,7 @@ __global__ __launch_bounds__(kThreads) void place_short_units_kernel(
     const int light_all = n_q - (heavy_before[f + n_q] - h0);              // light units of this queue
     const int light_me = (sidx - f) - (heavy_before[sidx] - h0);           // ... before this unit
     const bool is_light = heavy_before[sidx + 1] == heavy_before[sidx];
-    const int kept = max(0, light_all - ACCEL_TAIL_LIGHT);                 // light units that stay in line
+    const int kept = max(0, light_all - kTailLight);                 // light units that stay in line
     int pos;
     if (is_light && light_me >= kept)
         pos = n_q - (light_all - light_me);                                // held back: the last ones
@@ -858,9 +958,13 @@ __global__ __launch_bounds__(kThreads) void place_short_units_kernel(
 
 // Builds block4 from degrees given in partition order.  The output is a freshly
 // allocated device array (caller frees); *n_blocks is returned on the host.
+// The one synchronisation in here (the host has to know the number of blocks to allocate
+// them) also brings back, if asked, the blocks that precede row probe_row and the sorted
+// indptr at that row.  The emit kernel is left running on the stream.
 static int partition_device(Arena *tmp, const uint32_t *deg, const int32_t *s_indptr, int64_t rows,
                             int32_t **block4_out, int64_t *n_blocks, hipStream_t s,
-                            int64_t probe_row = -1, int64_t *blocks_before_probe = nullptr)
+                            int64_t probe_row = -1, int64_t *blocks_before_probe = nullptr,
+                            int64_t *nnz_before_probe = nullptr)
 {
     DevBuf head(tmp), cnt(tmp), sums(tmp), rb(tmp), b4;
     int rc;
@@ -877,17 +981,19 @@ static int partition_device(Arena *tmp, const uint32_t *deg, const int32_t *s_in
     if ((rc = device_scan<SumOp, false>(cnt.as<int>(), rows, rb.as<int>(), rb.as<int>() + rows,
                                         sums.as<int>(), s)))
         return rc;
-    int nb = 0, before = 0;
+    int nb = 0, before = 0, nnz_before = 0;
     ACCEL_HIP(hipMemcpyAsync(&nb, rb.as<int>() + rows, sizeof(int), hipMemcpyDeviceToHost, s));
     if (blocks_before_probe && probe_row >= 0 && probe_row <= rows)   // rb[rows] is the total
         ACCEL_HIP(hipMemcpyAsync(&before, rb.as<int>() + probe_row, sizeof(int), hipMemcpyDeviceToHost, s));
+    if (nnz_before_probe && probe_row >= 0 && probe_row <= rows)
+        ACCEL_HIP(hipMemcpyAsync(&nnz_before, s_indptr + probe_row, sizeof(int), hipMemcpyDeviceToHost, s));
     ACCEL_HIP(hipStreamSynchronize(s));
     if (blocks_before_probe) *blocks_before_probe = before;
+    if (nnz_before_probe) *nnz_before_probe = nnz_before;
     if ((rc = b4.alloc(sizeof(int4) * (size_t)nb))) return rc;
     emit_block4_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(
         deg, s_indptr, head.as<int>(), rb.as<int>(), rows, b4.as<int4>());
     ACCEL_HIP(hipGetLastError());
-    ACCEL_HIP(hipStreamSynchronize(s));
     *n_blocks = nb;
     *block4_out = static_cast<int32_t *>(b4.release());
     return ACCEL_OK;
@@ -906,7 +1012,7 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
     if ((rc = deg.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
     if ((rc = st.alloc(sizeof(Stats)))) return rc;
     ACCEL_HIP(hipMemsetAsync(st.p, 0, sizeof(Stats), s));
-    degree_kernel<<<dim3(std::min(grid_for(rows), 2048u)), dim3(kThreads), 0, s>>>(
+    degree_kernel<<<dim3(std::min(grid_for(rows), kDegreeGroups)), dim3(kThreads), 0, s>>>(
         indptr_dev, rows, nnz, deg.as<uint32_t>(), st.as<Stats>(), kDegBound, kDegBound);
     Stats hs;
     ACCEL_HIP(hipMemcpyAsync(&hs, st.p, sizeof(Stats), hipMemcpyDeviceToHost, s));
@@ -915,7 +1021,9 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
         set_error("indptr must start at 0, be non-decreasing and end at nnz");
         return ACCEL_ERR_CSR;
     }
-    return partition_device(&tmp, deg.as<uint32_t>(), indptr_dev, rows, block4_dev, n_blocks, s);
+    if ((rc = partition_device(&tmp, deg.as<uint32_t>(), indptr_dev, rows, block4_dev, n_blocks, s))) return rc;
+    ACCEL_HIP(hipStreamSynchronize(s));               // the temporaries go away with this scope
+    return ACCEL_OK;
 }
 
 // The launch plan.  One work unit per wavefront, kWavesPerGroup units per
@@ -1129,13 +1237,11 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
 //   208 k non-zeros, power law:        11.8 / 12.4 / 19.8 us  ->  7.9 / 10.5 / 12.6 us
 //   1.2 M, 1.6 M and 2.4 M non-zeros:  wavefront units are faster (26 / 53 / 99 us against
 //                                      34 / 55 / 102 us on the 1.2 M one).
-#ifndef ACCEL_TEAM_MAX_NNZ
-#define ACCEL_TEAM_MAX_NNZ (512 * 1024)
-#endif
+constexpr int64_t kTeamMaxNnz = 512 * 1024;
 static bool choose_plan_team(int64_t rows, int64_t nnz)
 {
     (void)rows;
-    return nnz < (int64_t)ACCEL_TEAM_MAX_NNZ;
+    return nnz < kTeamMaxNnz;
 }
 
 // Unit size of the launch plan: the most non-zeros of a unit of several whole rows (and,
@@ -1158,9 +1264,7 @@ static int choose_plan_unit(int64_t rows, int64_t nnz, bool team)
 // Measured with 384, 256, 192, 128 and 96 (N = 64): 192 is 8 % faster than 384 on the
 // dense 115 M-non-zero matrix, 2 % on the 125 M power-law one, neutral elsewhere;
 // below 192 the extra partial sums start to cost at N = 16.
-#ifndef ACCEL_PLAN_SPLIT
-#define ACCEL_PLAN_SPLIT 192
-#endif
+constexpr int kPlanSplit = 192;
 // Columns within this distance of a row's place on the diagonal count as near: 8,192 rows of
 // X of 64 floats are half of one L2.
 constexpr int kLocalityBand = 4096;
@@ -1169,7 +1273,7 @@ static int choose_plan_split(int64_t rows, int64_t nnz, bool team)
 {
     (void)rows;
     (void)nnz;
-    return team ? kDegBound : ACCEL_PLAN_SPLIT;        // workgroup units: rows up to one unit stay whole
+    return team ? kDegBound : kPlanSplit;        // workgroup units: rows up to one unit stay whole
 }
 
 // 64-bit content hash of n 4-byte words: the sum over i of mix(i, word i) modulo 2^64,
@@ -1239,9 +1343,9 @@ int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s)
         }
     }
     if (n_long > 0)
-        group_long_rows_kernel<<<dim3((unsigned)n_long), dim3(kThreads), 0, s>>>(
-            h->indptr, h->idx, h->val, h->perm, h->s_indptr, first_long, h->plan_groups,
-            sidx.as<int32_t>(), sval.as<float>(), nullptr);
+        launch_group_long_rows(h->indptr, h->idx, h->val, h->perm, h->s_indptr, first_long, n_long,
+                               std::min<int64_t>(h->n_wide_rows, n_long), h->plan_groups,
+                               sidx.as<int32_t>(), sval.as<float>(), nullptr, s);
     ACCEL_HIP(hipGetLastError());
     ACCEL_HIP(hipStreamSynchronize(s));
     h->s_idx = static_cast<int32_t *>(sidx.release());
@@ -1274,34 +1378,34 @@ int preprocess_device(accel_handle *h)
         return ACCEL_OK;
     }
 
-    // temporaries: about 40 bytes per row when the rows have to be sorted, 24 otherwise,
-    // plus what the split rows need; further chunks are added on demand
+    // temporaries: a small first chunk for the degrees and the statistics; once those are
+    // known, one chunk sized for everything that follows (see below)
     Arena tmp;
-    tmp.next_chunk = (size_t)rows * 44 + (size_t)(rows / kTile + 1) * 1100 + (1 << 20);
+    tmp.next_chunk = (size_t)rows * 4 + 4096;
     DevBuf deg(&tmp), st(&tmp);
     if ((rc = deg.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
     if ((rc = st.alloc(sizeof(Stats)))) return rc;
     ACCEL_HIP(hipMemsetAsync(st.p, 0, sizeof(Stats), s));
-    degree_kernel<<<dim3(std::min(grid_for(rows), 2048u)), dim3(kThreads), 0, s>>>(
+    degree_kernel<<<dim3(std::min(grid_for(rows), kDegreeGroups)), dim3(kThreads), 0, s>>>(
         h->indptr, rows, nnz, deg.as<uint32_t>(), st.as<Stats>(), h->plan_split, h->plan_unit);
+    // validation of the columns and the locality sample run in the same batch: both only read
+    // idx inside [0, nnz), whatever indptr holds
+    if (nnz > 0) {
+        const unsigned g = (unsigned)std::min<int64_t>((nnz / 4 + kThreads - 1) / kThreads + 1, 16384);
+        index_check_kernel<<<dim3(g), dim3(kThreads), 0, s>>>(h->idx, nnz, h->cols, st.as<Stats>());
+        locality_kernel<<<dim3(grid_for((rows + kLocalityStride - 1) / kLocalityStride)), dim3(kThreads), 0, s>>>(
+            h->indptr, h->idx, rows, h->cols, nnz, kLocalityBand, st.as<Stats>());
+    }
     Stats hs;
     ACCEL_HIP(hipMemcpyAsync(&hs, st.p, sizeof(Stats), hipMemcpyDeviceToHost, s));
     ACCEL_HIP(hipStreamSynchronize(s));
-    if (hs.bad_indptr) {   // checked before idx is touched: nnz is trusted from here on
+    if (hs.bad_indptr) {
         set_error("indptr must start at 0, be non-decreasing and end at nnz");
         return ACCEL_ERR_CSR;
     }
-    if (nnz > 0) {
-        const unsigned g = (unsigned)std::min<int64_t>((nnz + kThreads - 1) / kThreads, 65536);
-        index_check_kernel<<<dim3(g), dim3(kThreads), 0, s>>>(h->idx, nnz, h->cols, st.as<Stats>());
-        locality_kernel<<<dim3(grid_for((rows + kLocalityStride - 1) / kLocalityStride)), dim3(kThreads), 0, s>>>(
-            h->indptr, h->idx, rows, h->cols, kLocalityBand, st.as<Stats>());
-        ACCEL_HIP(hipMemcpyAsync(&hs, st.p, sizeof(Stats), hipMemcpyDeviceToHost, s));
-        ACCEL_HIP(hipStreamSynchronize(s));
-        if (hs.bad_index) {
-            set_error("a column index lies outside [0, cols)");
-            return ACCEL_ERR_CSR;
-        }
+    if (hs.bad_index) {
+        set_error("a column index lies outside [0, cols)");
+        return ACCEL_ERR_CSR;
     }
     // A matrix whose non-zeros lie near the diagonal keeps its locality only in rows that stay
     // whole (their neighbourhood of X is what a die has in its L2 while it works through a band
@@ -1321,7 +1425,14 @@ int preprocess_device(accel_handle *h)
     h->n_long_blocks = hs.n_long_blocks;
     h->n_split_rows = hs.n_split_rows;
     h->n_big_rows = hs.n_big_rows;
+    h->n_wide_rows = hs.n_wide_rows;
     h->identity_perm = !hs.unsorted;
+    // Everything else comes out of one more chunk: 12.5 bytes per row for the sort, 16 for
+    // the scans of the partition, up to 45 per whole-row unit of the plan (at most one per
+    // row), about 800 per split row (its 64 group counts and 120 bin slots).  A device
+    // allocation costs some 50 us whatever its size; a dozen of them were a sixth of the
+    // preprocessing time.
+    tmp.next_chunk = (size_t)rows * 76 + (size_t)hs.n_split_rows * 832 + ((size_t)2 << 20);
 
     // ---- degree sort ------------------------------------------------------
     uint32_t *sdeg = deg.as<uint32_t>();
@@ -1340,17 +1451,29 @@ int preprocess_device(accel_handle *h)
                                         sip.as<int>() + rows, ssums.as<int>(), s)))
         return rc;
 
+    // ---- partition ----------------------------------------------------------
+    // (before the sorted CSR: its one synchronisation also tells how many non-zeros the rows
+    // that are not split hold, which sizes the gather below)
+    const int64_t n_long = hs.n_split_rows, first_long = rows - n_long;
+    int32_t *b4 = nullptr;
+    int64_t nb = 0;
+    int64_t n_short_entries = 0;   // block4 entries of the rows that are not cut into pieces
+    int64_t nnz_short = 0;         // their non-zeros
+    if ((rc = partition_device(&tmp, sdeg, sip.as<int32_t>(), rows, &b4, &nb, s, first_long, &n_short_entries,
+                               &nnz_short)))
+        return rc;
+    h->block4 = b4;
+    h->n_blocks = nb;
+    if (nb + (int64_t)kMaxGroups * n_long + kXcds * kWavesPerGroup > (int64_t)INT_MAX) {
+        set_error("the launch plan would exceed 2^31 work units (%lld block4 entries)", (long long)nb);
+        return ACCEL_ERR_ARG;
+    }
+
     // ---- sorted CSR ---------------------------------------------------------
     // Split rows (more than plan_split non-zeros: the last n_long rows of the sorted
     // order) are stored grouped by column group; all other rows keep their non-zero
     // order.  The caller's arrays are used in place only when the input was already
     // sorted and has no split row.
-    const int64_t n_long = hs.n_split_rows, first_long = rows - n_long;
-    int32_t nnz_short32 = 0;                             // non-zeros of the rows that are not split
-    ACCEL_HIP(hipMemcpyAsync(&nnz_short32, sip.as<int32_t>() + first_long, sizeof(int32_t),
-                             hipMemcpyDeviceToHost, s));
-    ACCEL_HIP(hipStreamSynchronize(s));
-    const int64_t nnz_short = nnz_short32;
     const bool own_copy = !h->identity_perm || n_long > 0;
     DevBuf sidx, sval, permbuf, gcount(&tmp);
     if (own_copy) {
@@ -1375,25 +1498,11 @@ int preprocess_device(accel_handle *h)
         }
         if (n_long > 0) {
             if ((rc = gcount.alloc(sizeof(int) * (size_t)n_long * kMaxGroups))) return rc;
-            group_long_rows_kernel<<<dim3((unsigned)n_long), dim3(kThreads), 0, s>>>(
-                h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), first_long, h->plan_groups,
-                sidx.as<int32_t>(), sval.as<float>(), gcount.as<int>());
+            launch_group_long_rows(h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), first_long, n_long,
+                                   std::min<int64_t>(hs.n_wide_rows, n_long), h->plan_groups,
+                                   sidx.as<int32_t>(), sval.as<float>(), gcount.as<int>(), s);
         }
         ACCEL_HIP(hipGetLastError());
-    }
-
-    // ---- partition ----------------------------------------------------------
-    int32_t *b4 = nullptr;
-    int64_t nb = 0;
-    int64_t n_short_entries = 0;   // block4 entries of the rows that are not cut into pieces
-    if ((rc = partition_device(&tmp, sdeg, sip.as<int32_t>(), rows, &b4, &nb, s, first_long, &n_short_entries)))
-        return rc;
-    ACCEL_HIP(hipStreamSynchronize(s));
-    h->block4 = b4;
-    h->n_blocks = nb;
-    if (nb + (int64_t)kMaxGroups * n_long + kXcds * kWavesPerGroup > (int64_t)INT_MAX) {
-        set_error("the launch plan would exceed 2^31 work units (%lld block4 entries)", (long long)nb);
-        return ACCEL_ERR_ARG;
     }
 
     // ---- work list ------------------------------------------------------------

@@ -35,7 +35,7 @@ struct StateHeader {
     int64_t rows, cols, nnz;
     uint64_t hash_indptr, hash_idx;
     int64_t n_blocks, n_long_blocks, n_long_rows, n_zero_rows, n_units, n_long_units, n_split_rows,
-        n_big_rows;
+        n_big_rows, n_wide_rows;
     int32_t max_degree, identity_perm, plan_unit, plan_split, plan_groups, plan_team, local,
         waves_per_group;
     int64_t words[kNumArrays];        // 4-byte words of each stored array (0: absent)
@@ -131,7 +131,7 @@ int accel_save_state(const accel_handle *h, const char *path)
     hd.rows = h->rows; hd.cols = h->cols; hd.nnz = h->nnz;
     hd.n_blocks = h->n_blocks; hd.n_long_blocks = h->n_long_blocks; hd.n_long_rows = h->n_long_rows;
     hd.n_zero_rows = h->n_zero_rows; hd.n_units = h->n_units; hd.n_long_units = h->n_long_units;
-    hd.n_split_rows = h->n_split_rows; hd.n_big_rows = h->n_big_rows;
+    hd.n_split_rows = h->n_split_rows; hd.n_big_rows = h->n_big_rows; hd.n_wide_rows = h->n_wide_rows;
     hd.max_degree = h->max_degree; hd.identity_perm = h->identity_perm ? 1 : 0;
     hd.plan_unit = h->plan_unit; hd.plan_split = h->plan_split; hd.plan_groups = h->plan_groups;
     hd.plan_team = h->plan_team ? 1 : 0; hd.local = h->local ? 1 : 0;
@@ -204,7 +204,8 @@ int accel_load_state(accel_handle *h, const char *path)
                                       4 * hd.n_blocks, 4 * hd.n_units,
                                       hd.rows > 0 ? hd.n_split_rows + 1 : 0};
     bool sane = hd.n_blocks >= 0 && hd.n_units >= 0 && hd.n_split_rows >= 0 && hd.n_split_rows <= hd.rows &&
-                hd.n_big_rows >= 0 && hd.n_big_rows <= hd.n_split_rows && hd.n_zero_rows >= 0 &&
+                hd.n_big_rows >= 0 && hd.n_big_rows <= hd.n_split_rows && hd.n_wide_rows >= 0 &&
+                hd.n_wide_rows <= hd.rows && hd.n_zero_rows >= 0 &&
                 hd.n_zero_rows <= hd.rows && hd.n_long_units >= 0 && hd.n_long_units <= hd.n_units &&
                 hd.n_blocks <= hd.rows + hd.nnz && hd.n_units <= 0x7fffffffLL &&
                 hd.n_units % (kXcds * kWavesPerGroup) == 0 &&
@@ -270,7 +271,8 @@ int accel_load_state(accel_handle *h, const char *path)
     h->identity_perm = hd.identity_perm != 0;
     h->n_blocks = hd.n_blocks; h->n_long_blocks = hd.n_long_blocks; h->n_long_rows = hd.n_long_rows;
     h->n_zero_rows = hd.n_zero_rows; h->n_units = hd.n_units; h->n_long_units = hd.n_long_units;
-    h->n_split_rows = hd.n_split_rows; h->n_big_rows = hd.n_big_rows; h->max_degree = hd.max_degree;
+    h->n_split_rows = hd.n_split_rows; h->n_big_rows = hd.n_big_rows; h->n_wide_rows = hd.n_wide_rows;
+    h->max_degree = hd.max_degree;
     h->plan_unit = hd.plan_unit; h->plan_split = hd.plan_split; h->plan_groups = hd.plan_groups;
     h->plan_team = hd.plan_team != 0; h->local = hd.local != 0;
     // non-zeros of the rows that are not split = sorted indptr at the first split row

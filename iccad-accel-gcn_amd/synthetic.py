@@ -216,6 +216,71 @@ def hub_graph_small(seed=GRAPH_SEED, n=6_000, n_hubs=4, hub_lo=900, hub_hi=2_500
     return g
 
 
+# ----------------------------------------------------------------------------
+# graphs with the degree sequences of upstream's own benchmark set
+# ----------------------------------------------------------------------------
+def upstream_graph_names():
+    return sorted(_upstream_degrees())
+
+
+def _upstream_degrees():
+    import json
+    from pathlib import Path
+    return json.loads((Path(__file__).resolve().parent / "data" / "upstream_degrees.json").read_text())
+
+
+def upstream_degree_sequence(name):
+    """Row degrees (ascending) of one of upstream's 16 published graphs (README.md:42
+    lists them), as its block_level_meta/<name>.block4 file encodes them."""
+    runs = np.asarray(_upstream_degrees()[name], dtype=np.int64)
+    return np.repeat(runs[:, 0], runs[:, 1])
+
+
+def fixture_graph(name, seed=0, sigma=0):
+    """A graph with exactly the degree sequence of one of upstream's benchmark graphs, rows
+    in shuffled order, values GCN-normalised.  The real edge lists are a download that is
+    not available offline, so the columns are synthetic: uniform random (sigma = 0), or,
+    to model a vertex order with locality, row id + N(0, sigma) (duplicates inside a row
+    merge, so such a graph has slightly fewer non-zeros)."""
+    deg = upstream_degree_sequence(name)
+    n = deg.size
+    rng = np.random.default_rng(seed)
+    deg = rng.permutation(deg)
+    src = np.repeat(np.arange(n, dtype=np.int64), deg)
+    if sigma > 0:
+        dst = np.clip(src + np.rint(rng.standard_normal(src.size) * sigma).astype(np.int64), 0, n - 1)
+    else:
+        dst = rng.integers(0, n, size=src.size, dtype=np.int64)
+    indptr, indices = _csr_from_edges(src, dst, n, n)
+    return Graph(name, indptr, indices, _gcn_values(indptr, indices), n, n)
+
+
+def uniform_graph(n_rows, degree, n_cols, seed=0):
+    """Every row has `degree` non-zeros with columns uniform over n_cols (repeats
+    allowed): a probe of the gather rate for an X of a chosen size."""
+    rng = np.random.default_rng(seed)
+    indptr = (np.arange(n_rows + 1, dtype=np.int64) * degree).astype(np.int32)
+    indices = rng.integers(0, n_cols, size=n_rows * degree).astype(np.int32)
+    values = rng.random(n_rows * degree, dtype=np.float32)
+    return Graph(f"uniform:{n_rows}:{degree}:{n_cols}", indptr, indices, values, n_rows, n_cols)
+
+
+def workload(spec):
+    """cfg1..cfg5, fixture:<name>, local:<name>:<sigma> or uniform:<rows>:<degree>:<cols>."""
+    if spec in WORKLOADS:
+        return WORKLOADS[spec]()
+    kind, _, rest = spec.partition(":")
+    if kind == "fixture":
+        return fixture_graph(rest)
+    if kind == "local":
+        name, sigma = rest.rsplit(":", 1)
+        return fixture_graph(name, sigma=int(sigma))
+    if kind == "uniform":
+        n_rows, degree, n_cols = (int(v) for v in rest.split(":"))
+        return uniform_graph(n_rows, degree, n_cols)
+    raise ValueError(f"unknown workload {spec}")
+
+
 WORKLOADS = {"cfg1": cfg1, "cfg2": cfg2, "cfg3": cfg3, "cfg4": cfg4, "cfg5": cfg5}
 # column counts each workload is swept over; the first entry is the default
 WORKLOAD_N = {"cfg1": (32,), "cfg2": (64, 16, 32, 128), "cfg3": (64, 32, 128),

@@ -83,7 +83,7 @@ def test_column_counts_of_upstreams_sweep_on_cfg2(gpu, N):
 
 
 @pytest.mark.parametrize("N,panel", [(64, 32), (128, 32), (128, 64), (96, 32), (48, 16), (256, 128)])
-def test_column_panels(gpu, mixed, N, panel):
+def test_forced_column_panels(gpu, mixed, N, panel):
     """A run cut into column panels computes the same product (a narrower panel gives a row
     more lane groups, so the order of the additions may differ)."""
     g, op = mixed

@@ -67,30 +67,65 @@ def _bench_module():
     return mod
 
 
-def test_bench_fixture_graphs_keep_the_golden_degree_sequence(pkg):
-    """bench.py's fixture:<g> and local:<g>:<sigma> workloads: the degree sequence is the one
-    the golden .block4 file of <g> encodes; local columns stay near the row id."""
-    import sys, os
-    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+def test_packaged_degree_sequences_are_the_golden_ones(pkg):
+    """data/upstream_degrees.json against the golden .block4 files it was read from."""
     import block4_codec
     from oracle import partition_oracle as po
-    bench = _bench_module()
-    golden = block4_codec.load("pubmed")
-    want = np.sort(po.degrees_from_block4(golden))
-    g = bench.fixture_graph(pkg, "pubmed")
+    assert pkg.synthetic.upstream_graph_names() == block4_codec.names()
+    for name in block4_codec.names():
+        want = np.sort(po.degrees_from_block4(block4_codec.load(name)))
+        assert np.array_equal(pkg.synthetic.upstream_degree_sequence(name), want), name
+
+
+def test_fixture_graphs_keep_the_degree_sequence(pkg):
+    """fixture:<g> and local:<g>:<sigma> workloads: the degree sequence is the one upstream's
+    .block4 file of <g> encodes; local columns stay near the row id."""
+    syn = pkg.synthetic
+    want = syn.upstream_degree_sequence("pubmed")
+    g = syn.workload("fixture:pubmed")
     well_formed(g)
     # duplicates inside a row merge, so a row may fall slightly short of its target degree
     got = np.sort(np.diff(g.indptr))
     assert got.size == want.size and np.all(got <= want) and got.sum() >= 0.999 * want.sum()
-    loc = bench.fixture_graph(pkg, "pubmed", sigma=50)
+    loc = syn.workload("local:pubmed:50")
     well_formed(loc)
     rows = np.repeat(np.arange(loc.n_rows), np.diff(loc.indptr))
     assert np.percentile(np.abs(loc.indices - rows), 99) <= 3 * 50 + 1
     assert np.abs(g.indices - np.repeat(np.arange(g.n_rows), np.diff(g.indptr))).mean() > 1000
+    with pytest.raises(ValueError):
+        syn.workload("nothing:1")
 
 
-def test_bench_uniform_probe_graph(pkg):
-    bench = _bench_module()
-    g = bench.uniform_graph(pkg, 1000, 7, 300)
+def test_uniform_probe_graph(pkg):
+    g = pkg.synthetic.workload("uniform:1000:7:300")
     assert g.n_rows == 1000 and g.n_cols == 300 and g.nnz == 7000
     assert np.all(np.diff(g.indptr) == 7) and g.indices.min() >= 0 and g.indices.max() < 300
+
+
+def test_bench_workload_cache_and_traffic_record(pkg, tmp_path):
+    """bench.py keeps generated workloads between runs, and reports recorded HBM traffic only
+    when it was taken with the kernel sources that are running."""
+    import json
+    import os
+    bench = _bench_module()
+    g1, cached1 = bench.load_workload(pkg.synthetic, "cfg1", str(tmp_path))
+    g2, cached2 = bench.load_workload(pkg.synthetic, "cfg1", str(tmp_path))
+    assert not cached1 and cached2
+    assert np.array_equal(g1.indptr, g2.indptr) and np.array_equal(g1.indices, g2.indices)
+    assert np.array_equal(g1.values, g2.values) and (g1.n_rows, g1.n_cols) == (g2.n_rows, g2.n_cols)
+    assert bench.load_workload(pkg.synthetic, "cfg1", "")[1] is False
+    # every committed traffic entry names the sources it was measured with
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    entries = json.load(open(os.path.join(root, "profiles", "spmm_gather_traffic.json")))
+    now = bench.kernel_source_hash()
+    assert len(now) == 16
+    for key, e in entries.items():
+        if key.startswith("_"):
+            continue
+        wl, n = key.rsplit("/N", 1)
+        value, note = bench.recorded_traffic(wl, int(n))
+        if e.get("source_sha16") == now:
+            assert value == e["traffic_bytes"] and note is None
+        else:
+            assert value is None and "taken with kernel sources" in note
+    assert bench.recorded_traffic("cfg1", 7) == (None, "this workload was not profiled")
