@@ -197,6 +197,9 @@ def main():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="only run the plain copy kernel over this many MiB, --steps times "
                          "(known-size reference for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--panel", type=int, default=0, help="column-panel width (accel_set_plan_panel; 0 = the library's choice)")
+    ap.add_argument("--plan-split", type=int, default=0, help="rows above this many non-zeros are split (accel_set_plan_split; 0 = the library's choice)")
+    ap.add_argument("--plan-groups", type=int, default=0, help="column groups of split rows (accel_set_plan_groups; 0 = per row)")
     ap.add_argument("--cache-dir", default="/tmp/accelgcn_bench_cache",
                     help="where generated workloads are kept between runs ('' = do not keep them)")
     a = ap.parse_args()
@@ -252,9 +255,12 @@ def main():
     t0 = time.time()
     op = pkg.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols)
     t_upload = time.time() - t0
-    op.preprocess()
+    plan = {k: v for k, v in (("plan_split", a.plan_split), ("plan_groups", a.plan_groups)) if v}
+    op.preprocess(**plan)
     first_preprocess_ms = op.info.preprocess_ms      # includes loading the kernels into the GPU
-    op.preprocess()                                  # the same work again: what a second graph would cost
+    op.preprocess(**plan)                            # the same work again: what a second graph would cost
+    if a.panel:
+        op.set_panel(a.panel)
     info = op.info
     log(f"[bench] upload {t_upload * 1e3:.0f} ms, preprocess {info.preprocess_ms:.1f} ms: "
         f"blocks={info.n_blocks} long_rows={info.n_long_rows} long_blocks={info.n_long_blocks} "
@@ -305,6 +311,8 @@ def main():
     achieved = alg_bytes / (main_avg_ms * 1e-3) / 1e9
     achieved_all = alg_bytes / (float(np.mean(tot_ms)) * 1e-3) / 1e9
     traffic, traffic_note = recorded_traffic(a.workload, N)
+    if a.panel or a.plan_split or a.plan_groups:
+        traffic, traffic_note = None, "run with plan options: not the configuration that was profiled"
     result = {
         "metric": "SpMM GFLOP/s (2*nnz*N), fp32",
         "value": round(flops / (ms_per_step * 1e-3) / 1e9, 2),
@@ -318,7 +326,9 @@ def main():
                    "preprocess_ms": round(info.preprocess_ms, 2),
                    "preprocess_first_call_ms": round(first_preprocess_ms, 2),
                    "preprocess_from_cache_ms": round(from_cache_ms, 2),
-                   "reference_protocol_ms": round(ref_protocol_ms, 5)},
+                   "reference_protocol_ms": round(ref_protocol_ms, 5),
+                   "plan": {"split_nz": int(info.plan_split_nz), "groups": int(info.plan_groups),
+                            "unit_nz": int(info.plan_unit_nz), "panel": a.panel}},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": traffic,

@@ -28,11 +28,16 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
 
 void release_products(accel_handle *h)
 {
-    if (h->perm) (void)hipFree(h->perm);
-    if (h->s_indptr) (void)hipFree(h->s_indptr);
-    if (h->owns_sorted) {
-        if (h->s_idx) (void)hipFree(const_cast<int32_t *>(h->s_idx));
-        if (h->s_val) (void)hipFree(const_cast<float *>(h->s_val));
+    if (h->slab) {
+        (void)hipFree(h->slab);
+        h->slab = nullptr;
+    } else {
+        if (h->perm) (void)hipFree(h->perm);
+        if (h->s_indptr) (void)hipFree(h->s_indptr);
+        if (h->owns_sorted) {
+            if (h->s_idx) (void)hipFree(const_cast<int32_t *>(h->s_idx));
+            if (h->s_val) (void)hipFree(const_cast<float *>(h->s_val));
+        }
     }
     if (h->work) (void)hipFree(h->work);
     if (h->long_slot) (void)hipFree(h->long_slot);

@@ -87,6 +87,7 @@ struct accel_handle {
     const int32_t *s_idx = nullptr;   // [nnz]  (aliases idx when identity)
     const float *s_val = nullptr;     // [nnz]  (aliases val when identity)
     bool owns_sorted = false;
+    void *slab = nullptr;             // when set: perm, s_indptr and the owned s_idx / s_val live in this one allocation
     int32_t *block4 = nullptr;        // [4*n_blocks]  the .block4 metadata (upstream ABI)
     // launch plan derived from block4 (see preprocess.hip, "work list")
     int32_t *work = nullptr;          // [4*n_units] one int4 per wavefront

@@ -421,6 +421,11 @@ struct DevBuf {  // frees on scope exit; with an arena, the arena owns the memor
     void *release() { void *q = p; p = nullptr; return q; }   // only for buffers without an arena
 };
 
+struct DevView {  // a part of a larger allocation, with DevBuf's accessors
+    void *p = nullptr;
+    template <class T> T *as() { return static_cast<T *>(p); }
+};
+
 inline unsigned grid_for(int64_t n) { return (unsigned)((n + kThreads - 1) / kThreads); }
 // Workgroups of degree_kernel: each ends with a dozen atomics on the same few words, which
 // the memory system applies one after the other (2,048 workgroups: 160 us on 2.45 M rows,
@@ -474,35 +479,38 @@ int radix_sort_pairs(Arena *tmp, uint32_t *keys, int64_t n, uint32_t max_key, hi
 constexpr int kPermuteNz = 4;                        // non-zeros per thread
 constexpr int kPermuteTile = kThreads * kPermuteNz;  // non-zeros per workgroup
 
+// tile_first[t] = the sorted row that holds non-zero t * kPermuteTile of the sorted matrix,
+// for every tile that starts before n_take.  One thread per row: a row writes the entry of
+// every tile boundary that falls inside it (rows without non-zeros write none).
+__global__ __launch_bounds__(kThreads) void tile_first_kernel(const int32_t *__restrict__ s_indptr,
+                                                              int64_t rows, int64_t n_take,
+                                                              int *__restrict__ tile_first)
+{
+    const int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (r >= rows) return;
+    const int64_t a = s_indptr[r], b = min((int64_t)s_indptr[r + 1], n_take);
+    for (int64_t t = (a + kPermuteTile - 1) / kPermuteTile; t * kPermuteTile < b; t++) tile_first[t] = (int)r;
+}
+
 // A workgroup copies kPermuteTile consecutive non-zeros of the sorted matrix.  They belong
-// to at most kPermuteTile + 1 consecutive sorted rows (rows without non-zeros all precede
-// the first non-zero), whose boundaries and source offsets are put in LDS once; each
-// thread then finds the row of its non-zeros by a search in LDS.
+// to consecutive sorted rows, from tile_first[this tile] to tile_first[next tile] (at most
+// kPermuteTile + 1 rows, each but the first starting inside the tile), whose boundaries and
+// source offsets are put in LDS once; each thread then finds the row of its non-zeros by a
+// search in LDS.  last_row = the row that holds non-zero n_take - 1.
 __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
     const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
     const float *__restrict__ val, const int32_t *__restrict__ perm,
-    const int32_t *__restrict__ s_indptr, int64_t rows, int64_t n_take, int32_t *__restrict__ s_idx,
-    float *__restrict__ s_val)
+    const int32_t *__restrict__ s_indptr, const int *__restrict__ tile_first, int64_t last_row,
+    int64_t n_take, int32_t *__restrict__ s_idx, float *__restrict__ s_val)
 {
     __shared__ int row_end[kPermuteTile + 1];        // s_indptr[first + j + 1]
     __shared__ int64_t shift[kPermuteTile + 1];      // source position minus sorted position, per row
-    __shared__ int64_t first_row_s;
     const int64_t p0 = (int64_t)blockIdx.x * kPermuteTile;
     const int64_t p1 = min(p0 + kPermuteTile, n_take);   // this workgroup copies [p0, p1)
-    if (threadIdx.x == 0) {
-        int64_t lo = 0, hi = rows - 1;               // first row whose end is beyond p0
-        while (lo < hi) {
-            const int64_t mid = (lo + hi) >> 1;
-            if ((int64_t)s_indptr[mid + 1] > p0) hi = mid; else lo = mid + 1;
-        }
-        first_row_s = lo;
-    }
-    __syncthreads();
-    const int64_t first_row = first_row_s;
-    // rows first_row .. first_row + n_here - 1 cover [p0, p1): every one of them but the last ends
-    // inside the range, and each holds at least one non-zero, so n_here <= p1 - p0 + 1
-    const int n_max = (int)min((int64_t)kPermuteTile + 1, rows - first_row);
-    for (int j = threadIdx.x; j < n_max; j += kThreads) {
+    const int64_t first_row = tile_first[blockIdx.x];
+    const int64_t end_row = blockIdx.x + 1 < gridDim.x ? (int64_t)tile_first[blockIdx.x + 1] : last_row;
+    const int n_here = (int)min((int64_t)kPermuteTile + 1, end_row - first_row + 1);
+    for (int j = threadIdx.x; j < n_here; j += kThreads) {
         const int64_t r = first_row + j;
         row_end[j] = s_indptr[r + 1];
         shift[j] = (int64_t)indptr[perm ? perm[r] : r] - (int64_t)s_indptr[r];
@@ -512,7 +520,7 @@ __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
     for (int q = 0; q < kPermuteNz; q++) {
         const int64_t p = p0 + (int64_t)q * kThreads + threadIdx.x;
         if (p >= p1) break;
-        int lo = 0, hi = n_max - 1;                  // first j with row_end[j] > p
+        int lo = 0, hi = n_here - 1;                 // first j with row_end[j] > p
         while (lo < hi) {
             const int mid = (lo + hi) >> 1;
             if ((int64_t)row_end[mid] > p) hi = mid; else lo = mid + 1;
@@ -530,6 +538,8 @@ __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
 // One workgroup per split row; counts[lr*64 + g] receives the size of each group
 // (counts may be null).
 // ---------------------------------------------------------------------------
+constexpr int kGroupRound = 4;   // elements per thread between two barriers of group_long_rows_kernel
+
 __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
     const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
     const float *__restrict__ val, const int32_t *__restrict__ perm,
@@ -538,7 +548,8 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
 {
     __shared__ int cnt[kMaxGroups];
     __shared__ int base[kMaxGroups];
-    __shared__ int wave_cnt[2][kThreads / 64][kMaxGroups];
+    // members of each group per (sub-round, wavefront); two copies used in turn
+    __shared__ int wave_cnt[2][kGroupRound][kThreads / 64][kMaxGroups];
     const int64_t r = first_long_row + blockIdx.x;
     const int64_t src0 = indptr[perm ? perm[r] : r];
     const int64_t dst0 = s_indptr[r];
@@ -556,39 +567,58 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
         if (counts) counts[(int64_t)blockIdx.x * kMaxGroups + threadIdx.x] = cnt[threadIdx.x];
     }
     __syncthreads();
+    // A round places kGroupRound * 256 consecutive non-zeros; inside a round the order is
+    // sub-round, then wavefront, then lane, which is the order of the row (the result is the
+    // stable partition by group).  Long rows are a chain of rounds, so a round does as much
+    // as fits between its two barriers.
     int flip = 0;
-    for (int c0 = 0; c0 < d; c0 += kThreads, flip ^= 1) {
-        const int i = c0 + threadIdx.x;
-        const bool valid = i < d;
-        const int col = valid ? idx[src0 + i] : 0;
-        const float v = valid ? val[src0 + i] : 0.0f;
-        const int g = col_group(col, ng);
-        wave_cnt[flip][w][lane] = 0;                    // each wavefront clears its own row
-        // lanes of this wavefront with the same group
-        unsigned long long peers = __ballot(valid);
+    for (int c0 = 0; c0 < d; c0 += kGroupRound * kThreads, flip ^= 1) {
+        int col[kGroupRound], g[kGroupRound], rank[kGroupRound];
+        float v[kGroupRound];
+        bool valid[kGroupRound];
 #pragma unroll
-        for (int b = 0; b < 6; b++) {
-            const bool bit = (g >> b) & 1;
-            const unsigned long long bal = __ballot(bit);
-            peers &= bit ? bal : ~bal;
+        for (int e = 0; e < kGroupRound; e++) {
+            const int i = c0 + e * kThreads + (int)threadIdx.x;
+            valid[e] = i < d;
+            col[e] = valid[e] ? idx[src0 + i] : 0;
+            v[e] = valid[e] ? val[src0 + i] : 0.0f;
+            g[e] = col_group(col[e], ng);
+            wave_cnt[flip][e][w][lane] = 0;             // each wavefront clears its own rows
         }
-        const int rank = __popcll(peers & ((1ull << lane) - 1ull));
-        if (valid && rank == 0) wave_cnt[flip][w][g] = __popcll(peers);
+#pragma unroll
+        for (int e = 0; e < kGroupRound; e++) {
+            unsigned long long peers = __ballot(valid[e]);   // lanes of this wavefront with the same group
+#pragma unroll
+            for (int b = 0; b < 6; b++) {
+                const bool bit = (g[e] >> b) & 1;
+                const unsigned long long bal = __ballot(bit);
+                peers &= bit ? bal : ~bal;
+            }
+            rank[e] = __popcll(peers & ((1ull << lane) - 1ull));
+            if (valid[e] && rank[e] == 0) wave_cnt[flip][e][w][g[e]] = __popcll(peers);
+        }
         __syncthreads();
-        if (valid) {
-            int pos = base[g] + rank;
-            for (int q = 0; q < w; q++) pos += wave_cnt[flip][q][g];
-            s_idx[dst0 + pos] = col;
-            s_val[dst0 + pos] = v;
+#pragma unroll
+        for (int e = 0; e < kGroupRound; e++) {
+            if (!valid[e]) continue;
+            int pos = base[g[e]] + rank[e];
+            for (int e2 = 0; e2 < e; e2++)
+#pragma unroll
+                for (int q = 0; q < kThreads / 64; q++) pos += wave_cnt[flip][e2][q][g[e]];
+            for (int q = 0; q < w; q++) pos += wave_cnt[flip][e][q][g[e]];
+            s_idx[dst0 + pos] = col[e];
+            s_val[dst0 + pos] = v[e];
         }
         __syncthreads();
         if ((int)threadIdx.x < kMaxGroups) {
             int add = 0;
 #pragma unroll
-            for (int q = 0; q < kThreads / 64; q++) add += wave_cnt[flip][q][threadIdx.x];
+            for (int e = 0; e < kGroupRound; e++)
+#pragma unroll
+                for (int q = 0; q < kThreads / 64; q++) add += wave_cnt[flip][e][q][threadIdx.x];
             base[threadIdx.x] += add;
         }
-        // the next round uses the other half of wave_cnt and reads base only after
+        // the next round uses the other copy of wave_cnt and reads base only after
         // its own barrier, so no third barrier is needed here
     }
 }
@@ -653,6 +683,19 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_wave_kernel(
         }
         __builtin_amdgcn_wave_barrier();
     }
+}
+
+// Gathers the first n_take non-zeros of the sorted matrix (the rows before first_long)
+// from the caller's arrays through perm.  tile_first: n_take / kPermuteTile + 2 ints.
+static void launch_permute_csr(const int32_t *indptr, const int32_t *idx, const float *val,
+                               const int32_t *perm, const int32_t *s_indptr, int64_t rows,
+                               int64_t first_long, int64_t n_take, int *tile_first, int32_t *s_idx,
+                               float *s_val, hipStream_t s)
+{
+    if (n_take <= 0) return;
+    tile_first_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(s_indptr, rows, n_take, tile_first);
+    permute_csr_kernel<<<dim3((unsigned)((n_take + kPermuteTile - 1) / kPermuteTile)), dim3(kThreads), 0, s>>>(
+        indptr, idx, val, perm, s_indptr, tile_first, first_long - 1, n_take, s_idx, s_val);
 }
 
 // Regroups the n_long split rows (the last rows of the sorted order, ascending by
@@ -1328,7 +1371,7 @@ int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s)
         h->owns_sorted = false;
         return ACCEL_OK;
     }
-    DevBuf sidx, sval;
+    DevBuf sidx, sval, tiles;
     int rc;
     if ((rc = sidx.alloc(sizeof(int32_t) * (size_t)nnz))) return rc;
     if ((rc = sval.alloc(sizeof(float) * (size_t)nnz))) return rc;
@@ -1337,9 +1380,9 @@ int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s)
             ACCEL_HIP(hipMemcpyAsync(sidx.p, h->idx, sizeof(int32_t) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
             ACCEL_HIP(hipMemcpyAsync(sval.p, h->val, sizeof(float) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
         } else {
-            permute_csr_kernel<<<dim3((unsigned)((nnz_short + kPermuteTile - 1) / kPermuteTile)), dim3(kThreads), 0, s>>>(
-                h->indptr, h->idx, h->val, h->perm, h->s_indptr, rows, nnz_short, sidx.as<int32_t>(),
-                sval.as<float>());
+            if ((rc = tiles.alloc(sizeof(int) * (size_t)(nnz_short / kPermuteTile + 2)))) return rc;
+            launch_permute_csr(h->indptr, h->idx, h->val, h->perm, h->s_indptr, rows, first_long, nnz_short,
+                               tiles.as<int>(), sidx.as<int32_t>(), sval.as<float>(), s);
         }
     }
     if (n_long > 0)
@@ -1432,7 +1475,7 @@ int preprocess_device(accel_handle *h)
     // row), about 800 per split row (its 64 group counts and 120 bin slots).  A device
     // allocation costs some 50 us whatever its size; a dozen of them were a sixth of the
     // preprocessing time.
-    tmp.next_chunk = (size_t)rows * 76 + (size_t)hs.n_split_rows * 832 + ((size_t)2 << 20);
+    tmp.next_chunk = (size_t)rows * 76 + (size_t)hs.n_split_rows * 832 + (size_t)nnz / 256 + ((size_t)2 << 20);
 
     // ---- degree sort ------------------------------------------------------
     uint32_t *sdeg = deg.as<uint32_t>();
@@ -1443,9 +1486,26 @@ int preprocess_device(accel_handle *h)
             return rc;
     }
 
+    // ---- the products that stay: one allocation for the sorted indptr, the permutation
+    // and the sorted copy of the non-zeros (a device allocation costs some 50 us)
+    const int64_t n_long = hs.n_split_rows, first_long = rows - n_long;
+    const bool own_copy = !h->identity_perm || n_long > 0;
+    auto pad = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const size_t b_sip = pad(sizeof(int32_t) * (size_t)(rows + 1));
+    const size_t b_perm = h->identity_perm ? 0 : pad(sizeof(int32_t) * (size_t)rows);
+    const size_t b_nz = own_copy ? pad(sizeof(int32_t) * (size_t)nnz) : 0;
+    DevBuf slab;
+    if ((rc = slab.alloc(b_sip + b_perm + 2 * b_nz))) return rc;
+    DevView sip, permbuf, sidx, sval;                // parts of the slab
+    sip.p = slab.p;
+    if (b_perm) permbuf.p = slab.as<char>() + b_sip;
+    if (b_nz) {
+        sidx.p = slab.as<char>() + b_sip + b_perm;
+        sval.p = slab.as<char>() + b_sip + b_perm + b_nz;
+    }
+
     // ---- sorted indptr ------------------------------------------------------
-    DevBuf sip, ssums(&tmp);
-    if ((rc = sip.alloc(sizeof(int32_t) * (size_t)(rows + 1)))) return rc;
+    DevBuf ssums(&tmp);
     if ((rc = ssums.alloc(sizeof(int) * (size_t)(rows / kTile + 4)))) return rc;
     if ((rc = device_scan<SumOp, false>(reinterpret_cast<const int *>(sdeg), rows, sip.as<int>(),
                                         sip.as<int>() + rows, ssums.as<int>(), s)))
@@ -1454,7 +1514,6 @@ int preprocess_device(accel_handle *h)
     // ---- partition ----------------------------------------------------------
     // (before the sorted CSR: its one synchronisation also tells how many non-zeros the rows
     // that are not split hold, which sizes the gather below)
-    const int64_t n_long = hs.n_split_rows, first_long = rows - n_long;
     int32_t *b4 = nullptr;
     int64_t nb = 0;
     int64_t n_short_entries = 0;   // block4 entries of the rows that are not cut into pieces
@@ -1474,11 +1533,8 @@ int preprocess_device(accel_handle *h)
     // order) are stored grouped by column group; all other rows keep their non-zero
     // order.  The caller's arrays are used in place only when the input was already
     // sorted and has no split row.
-    const bool own_copy = !h->identity_perm || n_long > 0;
-    DevBuf sidx, sval, permbuf, gcount(&tmp);
+    DevBuf gcount(&tmp), tiles(&tmp);
     if (own_copy) {
-        if ((rc = sidx.alloc(sizeof(int32_t) * (size_t)nnz))) return rc;
-        if ((rc = sval.alloc(sizeof(float) * (size_t)nnz))) return rc;
         const int32_t *pm = reinterpret_cast<const int32_t *>(perm);
         if (h->identity_perm) {
             if (nnz_short > 0) {
@@ -1488,11 +1544,11 @@ int preprocess_device(accel_handle *h)
                                          hipMemcpyDeviceToDevice, s));
             }
         } else {
-            if (nnz_short > 0)
-                permute_csr_kernel<<<dim3((unsigned)((nnz_short + kPermuteTile - 1) / kPermuteTile)), dim3(kThreads), 0, s>>>(
-                    h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), rows, nnz_short,
-                    sidx.as<int32_t>(), sval.as<float>());
-            if ((rc = permbuf.alloc(sizeof(int32_t) * (size_t)rows))) return rc;
+            if (nnz_short > 0) {
+                if ((rc = tiles.alloc(sizeof(int) * (size_t)(nnz_short / kPermuteTile + 2)))) return rc;
+                launch_permute_csr(h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), rows, first_long, nnz_short,
+                                   tiles.as<int>(), sidx.as<int32_t>(), sval.as<float>(), s);
+            }
             ACCEL_HIP(hipMemcpyAsync(permbuf.p, perm, sizeof(int32_t) * (size_t)rows,
                                      hipMemcpyDeviceToDevice, s));
         }
@@ -1509,16 +1565,16 @@ int preprocess_device(accel_handle *h)
     if ((rc = build_work_list(&tmp, h, gcount.as<int>(), sip.as<int32_t>(), first_long, n_short_entries, perm, s)))
         return rc;
 
-    h->s_indptr = static_cast<int32_t *>(sip.release());
+    h->slab = slab.release();
+    h->s_indptr = sip.as<int32_t>();
+    h->perm = permbuf.as<int32_t>();                 // null for sorted input
     if (!own_copy) {
-        h->perm = nullptr;
         h->s_idx = h->idx;
         h->s_val = h->val;
         h->owns_sorted = false;
     } else {
-        h->perm = static_cast<int32_t *>(permbuf.release());   // stays null for sorted input
-        h->s_idx = static_cast<int32_t *>(sidx.release());
-        h->s_val = static_cast<float *>(sval.release());
+        h->s_idx = sidx.as<int32_t>();
+        h->s_val = sval.as<float>();
         h->owns_sorted = true;
     }
     h->ready = true;

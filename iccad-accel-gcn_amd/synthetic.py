@@ -281,6 +281,32 @@ def workload(spec):
     raise ValueError(f"unknown workload {spec}")
 
 
+def export_upstream_layout(spec_or_graph, graphs_dir, name=None):
+    """Write a workload the way upstream's programs read their datasets (main.cu:62-63,
+    block_level_partition.py:26-32): ``<name>.config`` (presence only), ``<name>.new_indptr``
+    and ``<name>.new_indices`` as raw little-endian int32, rows in ascending degree order
+    (ties keep their order).  Values are not part of the layout (upstream fills ones,
+    main.cu:114).  The adjacency must be square.  Returns the stem written."""
+    from pathlib import Path
+    g = workload(spec_or_graph) if isinstance(spec_or_graph, str) else spec_or_graph
+    if g.n_rows != g.n_cols:
+        raise ValueError("upstream's layout assumes a square adjacency")
+    name = name or g.name.replace(":", "-")
+    deg = np.diff(g.indptr).astype(np.int64)
+    perm = np.argsort(deg, kind="stable")
+    sip = np.zeros(g.n_rows + 1, dtype=np.int64)
+    np.cumsum(deg[perm], out=sip[1:])
+    # gather the rows in the new order
+    starts = g.indptr[:-1].astype(np.int64)[perm]
+    src = np.repeat(starts - sip[:-1], deg[perm]) + np.arange(int(sip[-1]), dtype=np.int64)
+    out = Path(graphs_dir)
+    out.mkdir(parents=True, exist_ok=True)
+    (out / f"{name}.config").write_text("")
+    sip.astype("<i4").tofile(out / f"{name}.new_indptr")
+    g.indices[src].astype("<i4").tofile(out / f"{name}.new_indices")
+    return name
+
+
 WORKLOADS = {"cfg1": cfg1, "cfg2": cfg2, "cfg3": cfg3, "cfg4": cfg4, "cfg5": cfg5}
 # column counts each workload is swept over; the first entry is the default
 WORKLOAD_N = {"cfg1": (32,), "cfg2": (64, 16, 32, 128), "cfg3": (64, 32, 128),

@@ -129,3 +129,18 @@ def test_bench_workload_cache_and_traffic_record(pkg, tmp_path):
         else:
             assert value is None and "taken with kernel sources" in note
     assert bench.recorded_traffic("cfg1", 7) == (None, "this workload was not profiled")
+
+
+def test_export_in_upstreams_layout(pkg, tmp_path):
+    """<name>.config / .new_indptr / .new_indices: degree-sorted rows, raw int32, the same matrix."""
+    from oracle import partition_oracle as po
+    syn = pkg.synthetic
+    g = syn.workload("fixture:pubmed")
+    name = syn.export_upstream_layout(g, tmp_path / "graphs")
+    assert name == "pubmed" and (tmp_path / "graphs" / "pubmed.config").exists()
+    ip = np.fromfile(tmp_path / "graphs" / "pubmed.new_indptr", dtype="<i4")
+    ix = np.fromfile(tmp_path / "graphs" / "pubmed.new_indices", dtype="<i4")
+    perm = po.degree_sort(g.indptr)
+    sip, six, _ = po.permute_csr(g.indptr, g.indices, g.values, perm)
+    assert np.array_equal(ip, sip) and np.array_equal(ix, six)
+    assert np.all(np.diff(np.diff(ip)) >= 0)
