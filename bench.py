@@ -200,6 +200,9 @@ def main():
     ap.add_argument("--panel", type=int, default=0, help="column-panel width (accel_set_plan_panel; 0 = the library's choice)")
     ap.add_argument("--plan-split", type=int, default=0, help="rows above this many non-zeros are split (accel_set_plan_split; 0 = the library's choice)")
     ap.add_argument("--plan-groups", type=int, default=0, help="column groups of split rows (accel_set_plan_groups; 0 = per row)")
+    ap.add_argument("--ld", type=int, default=0,
+                    help="also time accel_run_strided with rows of X and Y this many floats apart (>= N), "
+                         "on the host clock; reported as config.strided")
     ap.add_argument("--cache-dir", default="/tmp/accelgcn_bench_cache",
                     help="where generated workloads are kept between runs ('' = do not keep them)")
     a = ap.parse_args()
@@ -305,6 +308,23 @@ def main():
         ref_protocol += time.perf_counter() - t1
     ref_protocol_ms = ref_protocol / 4 * 1e3
 
+    strided = None
+    if a.ld:
+        if a.ld < N:
+            sys.exit("bench.py: --ld must be at least N")
+        sX, sY = pkg.DeviceBuffer(g.n_cols * a.ld * 4), pkg.DeviceBuffer(g.n_rows * a.ld * 4)
+        sX.fill_u32(0x3F000000)
+        for _ in range(3):
+            op.run_strided(sX, sY, N, a.ld)
+        op.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(a.steps):
+            op.run_strided(sX, sY, N, a.ld)
+        op.synchronize()
+        strided = {"ld": a.ld, "ms_per_step": round((time.perf_counter() - t1) / a.steps * 1e3, 5)}
+        sX.close()
+        sY.close()
+
     flops = 2.0 * g.nnz * N
     alg_bytes = g.nnz * 8 + g.n_cols * N * 4 + g.n_rows * N * 4
     main_avg_ms = float(np.mean(main_ms))
@@ -341,6 +361,8 @@ def main():
     }
     if traffic_note:
         result["roofline"]["traffic_stale"] = traffic_note
+    if strided:
+        result["config"]["strided"] = strided
 
     if a.compare_rocsparse:
         rs, Yr = rocsparse_baseline(pkg, op, g, dX, N)

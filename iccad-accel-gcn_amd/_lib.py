@@ -81,6 +81,7 @@ SIGNATURES = {
     "accel_get_perm": (C.c_int, [vp, i32p, C.c_int64]),
     "accel_get_sorted_csr": (C.c_int, [vp, i32p, i32p, f32p]),
     "accel_run": (C.c_int, [vp, vp, vp, C.c_int32, vp]),
+    "accel_run_strided": (C.c_int, [vp, vp, vp, C.c_int32, C.c_int32, vp]),
     "accel_reserve": (C.c_int, [vp, C.c_int32]),
     "accel_run_static": (C.c_int, [vp, vp, vp, C.c_int32, vp]),
     "accel_run_epilogue": (C.c_int, [vp, vp, vp, C.c_int32, vp, C.c_int, vp]),

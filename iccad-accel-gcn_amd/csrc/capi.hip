@@ -98,15 +98,20 @@ static int check_operand(accel_handle *h, const void *p, size_t bytes, const cha
 }
 
 // argument checks shared by the run entry points
-static int check_run(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias, const char *fn)
+static int check_run(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias, const char *fn,
+                     int32_t ld = 0)
 {
     if (!h) { set_error("%s: null handle", fn); return ACCEL_ERR_ARG; }
     if (!h->ready) { set_error("%s: call accel_preprocess first", fn); return ACCEL_ERR_STATE; }
     if (N <= 0) { set_error("%s: N must be positive, got %d", fn, N); return ACCEL_ERR_ARG; }
     if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("%s: null dense operand", fn); return ACCEL_ERR_ARG; }
     if (h->rows == 0) return ACCEL_OK;
-    if (int rc = check_operand(h, X, (size_t)h->cols * (size_t)N * sizeof(float), fn, "X")) return rc;
-    if (int rc = check_operand(h, Y, (size_t)h->rows * (size_t)N * sizeof(float), fn, "Y")) return rc;
+    if (ld <= 0) ld = N;
+    // the last row only has to hold N floats
+    const size_t x_floats = h->cols > 0 ? (size_t)(h->cols - 1) * (size_t)ld + (size_t)N : 0;
+    const size_t y_floats = (size_t)(h->rows - 1) * (size_t)ld + (size_t)N;
+    if (int rc = check_operand(h, X, x_floats * sizeof(float), fn, "X")) return rc;
+    if (int rc = check_operand(h, Y, y_floats * sizeof(float), fn, "Y")) return rc;
     return check_operand(h, bias, (size_t)N * sizeof(float), fn, "bias");
 }
 
@@ -622,6 +627,14 @@ int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream
     clear_error();
     if (int rc = check_run(h, X, Y, N, nullptr, "accel_run")) return rc;
     return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr);
+}
+
+int accel_run_strided(accel_handle *h, const float *X, float *Y, int32_t N, int32_t ld, void *stream)
+{
+    clear_error();
+    if (ld < N) { set_error("accel_run_strided: the row stride (%d) must be at least N (%d)", ld, N); return ACCEL_ERR_ARG; }
+    if (int rc = check_run(h, X, Y, N, nullptr, "accel_run_strided", ld)) return rc;
+    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, nullptr, 0, false, ld);
 }
 
 int accel_reserve(accel_handle *h, int32_t max_N)

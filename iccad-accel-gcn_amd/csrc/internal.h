@@ -134,7 +134,7 @@ void release_products(accel_handle *h);
 // spmm.hip
 int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
                 hipEvent_t after_main, const float *bias = nullptr, int relu = 0,
-                bool static_partial = false);
+                bool static_partial = false, int ld = 0);
 int reserve_partial(accel_handle *h, size_t floats);
 int fill_u32(void *dst, uint32_t v, size_t n, hipStream_t s);
 int copy_u32(void *dst, const void *src, size_t n, hipStream_t s);

@@ -436,8 +436,9 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
 __global__ __launch_bounds__(kReduceThreads) void long_row_reduce_kernel(
     const float *__restrict__ partial, const int32_t *__restrict__ long_slot,
     const int32_t *__restrict__ perm, int64_t first_split_row, int n_shared_rows, int n_shared_groups,
-    int rpw, int n_rows, float *__restrict__ Y, int N, const float *__restrict__ bias, int relu)
+    int rpw, int n_rows, float *__restrict__ Y, int N, int ld, const float *__restrict__ bias, int relu)
 {
+    // N columns; rows of Y and of the partial sums are ld floats apart
     __shared__ float red[kReduceThreads];
     const bool shared_group = (int)blockIdx.x < n_shared_groups;
     const int T = shared_group ? kReduceThreads / rpw : kReduceThreads;   // threads per row
@@ -447,7 +448,7 @@ __global__ __launch_bounds__(kReduceThreads) void long_row_reduce_kernel(
     const bool row_ok = lr < (shared_group ? n_shared_rows : n_rows);
     const int first = row_ok ? long_slot[lr] : 0;
     const int nseg = row_ok ? long_slot[lr + 1] - first : 0;
-    const float *src = partial + (int64_t)first * N;
+    const float *src = partial + (int64_t)first * ld;
     const int64_t r = first_split_row + lr;
     const int64_t out_row = row_ok ? (perm ? perm[r] : r) : 0;
     int cw = 1;                                    // columns per pass: power of two <= T
@@ -462,11 +463,11 @@ __global__ __launch_bounds__(kReduceThreads) void long_row_reduce_kernel(
             for (; sgm + 7 * sg < nseg; sgm += 8 * sg) {       // eight loads in flight, added in order
                 float v[8];
 #pragma unroll
-                for (int u = 0; u < 8; u++) v[u] = src[(int64_t)(sgm + u * sg) * N + c];
+                for (int u = 0; u < 8; u++) v[u] = src[(int64_t)(sgm + u * sg) * ld + c];
 #pragma unroll
                 for (int u = 0; u < 8; u++) acc += v[u];
             }
-            for (; sgm < nseg; sgm += sg) acc += src[(int64_t)sgm * N + c];
+            for (; sgm < nseg; sgm += sg) acc += src[(int64_t)sgm * ld + c];
         }
         red[threadIdx.x] = acc;
         __syncthreads();
@@ -475,7 +476,7 @@ __global__ __launch_bounds__(kReduceThreads) void long_row_reduce_kernel(
             for (int q = 1; q < sg; q++) sum += red[sub_row * T + q * cw + c_in];
             if (bias) sum += bias[c];
             if (relu) sum = fmaxf(sum, 0.0f);
-            Y[out_row * N + c] = sum;
+            Y[out_row * ld + c] = sum;
         }
         __syncthreads();
     }
@@ -620,16 +621,17 @@ int reserve_partial(accel_handle *h, size_t floats)
 }
 
 int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
-                hipEvent_t after_main, const float *bias, int relu, bool static_partial)
+                hipEvent_t after_main, const float *bias, int relu, bool static_partial, int ld)
 {
     if (h->rows == 0) return ACCEL_OK;
+    if (ld <= 0) ld = N;                             // rows of X and Y are ld floats apart
     // 16-byte vectors whenever a row holds one.  When N is not a multiple of 4, or X or Y
     // is not 16-byte aligned, rows start at odd multiples of 4 bytes: the vectors are then
     // loaded and stored at 4-byte aligned addresses, and a row's last vector is moved back
     // so that it ends with the row (it overlaps the one before; both lanes hold the same
     // sums for the shared columns).  Scalar lanes are left for N < 4.
     const uintptr_t align = reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Y);
-    const int mode = N < 4 ? 2 : (N % 4 == 0 && align % 16 == 0) ? 0 : 1;
+    const int mode = N < 4 ? 2 : (N % 4 == 0 && ld % 4 == 0 && align % 16 == 0) ? 0 : 1;
     const int vec = mode == 2 ? 1 : 4;
 
     // partial sums of the pieces of split rows: the handle's buffer (allocated here when a
@@ -638,7 +640,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     bool guard_partial = false;
     if (static_partial) {
         partial = nullptr;
-        const size_t need = (size_t)h->n_long_units * (size_t)N;
+        const size_t need = (size_t)h->n_long_units * (size_t)ld;
         if (need > kStaticScratchFloats) {
             set_error("accel_run_static: this matrix needs %zu floats of partial sums at N = %d "
                       "(%lld pieces of split rows x N), the static scratch holds %zu",
@@ -662,7 +664,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
             return ACCEL_ERR_STATE;
         }
         (void)hipGetLastError();
-        const size_t need = (size_t)h->n_long_units * (size_t)N;
+        const size_t need = (size_t)h->n_long_units * (size_t)ld;
         if (h->partial_floats < need) {
             if (capturing) {
                 set_error("the partial-sum buffer has to grow for N = %d and the stream is capturing: "
@@ -688,7 +690,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         (forced || (h->nnz >= kPanelMinNnz && h->nnz >= 16 * h->rows)))
         panel = want;
     // operands below 4 GiB are addressed with 32-bit byte offsets (see gather_row)
-    const bool wide = (uint64_t)h->cols * (uint64_t)N * 4u > 0xFFFFFFFFull;
+    const bool wide = (uint64_t)h->cols * (uint64_t)ld * 4u > 0xFFFFFFFFull;
     const int4 *wk = reinterpret_cast<const int4 *>(h->work);
     const int64_t entry_groups = h->plan_team ? h->n_units : h->n_units / kWaves;
     for (int c0 = 0; c0 < N; c0 += panel) {
@@ -711,7 +713,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         float *Yp = Y + c0, *Pp = partial ? partial + c0 : nullptr;
         const float *bp = bias ? bias + c0 : nullptr;
         const LaunchArgs la{h->plan_team, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                            Xp, Yp, Pp, n, N, (int)h->n_zero_rows, (int)zero_groups, bp, relu};
+                            Xp, Yp, Pp, n, ld, (int)h->n_zero_rows, (int)zero_groups, bp, relu};
         const int rc = launch_for_mode(mode, wide, L, la);
         if (rc) return rc;
     }
@@ -724,7 +726,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         const int shared_groups = (n_shared + rpw - 1) / rpw;
         long_row_reduce_kernel<<<dim3((unsigned)(shared_groups + n_big)), dim3(kReduceThreads), 0, stream>>>(
             partial, h->long_slot, h->perm, h->rows - h->n_split_rows, n_shared, shared_groups, rpw,
-            n_split, Y, N, bias, relu);
+            n_split, Y, N, ld, bias, relu);
     }
     ACCEL_HIP(hipGetLastError());
     if (guard_partial) {

@@ -153,6 +153,16 @@ class AccelSpMM:
         x, y, _ = self._operands(X, Y, N)
         check(lib().accel_run(self._h, x, y, int(N), ptr(stream)))
 
+    def run_strided(self, X, Y, N: int, ld: int, stream=None) -> None:
+        """``run`` on operands whose rows are ``ld`` >= N floats apart (see accel_run_strided):
+        rows of X padded to a multiple of 32 floats touch fewer cache lines per gather."""
+        N, ld = int(N), int(ld)
+        if N <= 0 or ld < N:
+            raise AccelError(_lib.ERR_ARG, f"need 0 < N <= ld, got N={N}, ld={ld}")
+        x = _lib.dev_ptr(X, ((self.n_cols - 1) * ld + N) * 4 if self.n_cols else 0, "X")
+        y = _lib.dev_ptr(Y, ((self.n_rows - 1) * ld + N) * 4 if self.n_rows else 0, "Y")
+        check(lib().accel_run_strided(self._h, x, y, N, ld, ptr(stream)))
+
     def reserve(self, max_N: int) -> None:
         """Allocate the partial-sum buffer for every N up to ``max_N`` now, so that no later
         run allocates (see accel_reserve)."""

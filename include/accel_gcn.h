@@ -226,6 +226,16 @@ int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream
 int accel_run_epilogue(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias,
                        int flags, void *stream);
 
+/* accel_run on operands whose rows are `ld` floats apart (ld >= N; accel_run is ld = N,
+ * the only layout upstream's kernel knows: it indexes row * feat_in + lane,
+ * spmm_accel.cu:75,84).  What it is for: the time of a run is set by the 128-byte lines a
+ * gathered row of X touches.  Rows of N = 127 floats packed back to back straddle five
+ * lines each, padded to ld = 128 they touch four; N = 50 at ld = 64 two instead of two and
+ * a half.  A caller that keeps X padded to a multiple of 32 floats gets the time of the
+ * next multiple for any N.  The columns N .. ld-1 of X are never read and those of Y never
+ * written.  The partial-sum buffer is sized for ld (accel_reserve(h, ld)). */
+int accel_run_strided(accel_handle *h, const float *X, float *Y, int32_t N, int32_t ld, void *stream);
+
 /* accel_run keeps the partial sums of split rows (pieces x N floats) in a buffer of the
  * handle.  It is allocated by the first accel_run with a given N and replaced by a larger
  * one when a later run brings a larger N; a HIP graph captured with the old buffer must

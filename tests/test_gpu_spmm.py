@@ -68,6 +68,31 @@ def test_operands_at_any_4_byte_alignment(gpu, mixed, N):
         dY.close()
 
 
+@pytest.mark.parametrize("N,ld", [(127, 128), (50, 64), (64, 80), (17, 32), (3, 8), (130, 131), (300, 320)])
+def test_rows_with_a_stride(gpu, mixed, N, ld):
+    """accel_run_strided: rows of X and Y are ld floats apart; the padding columns of X are
+    never read (they hold NaN) and those of Y never written."""
+    g, op = mixed
+    X = np.random.default_rng(N).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    Xp = np.full((g.n_cols, ld), np.nan, np.float32)
+    Xp[:, :N] = X
+    dX = gpu.DeviceBuffer.from_numpy(Xp.reshape(-1)[: (g.n_cols - 1) * ld + N])   # no padding behind the last row
+    dY = gpu.DeviceBuffer(((g.n_rows - 1) * ld + N) * 4)
+    dY.fill_u32(0x7FC00000)
+    op.run_strided(dX, dY, N, ld)
+    op.synchronize()
+    flat = dY.to_numpy(np.float32, ((g.n_rows - 1) * ld + N,))
+    Yp = np.full((g.n_rows, ld), np.nan, np.float32)
+    Yp.reshape(-1)[: flat.size] = flat
+    assert np.isfinite(Yp[:, :N]).all()
+    assert np.isnan(Yp[:-1, N:]).all(), "padding columns of Y were written"
+    assert so.check(np.ascontiguousarray(Yp[:, :N]), g.indptr, g.indices, g.values, X) <= TOL
+    with pytest.raises(gpu.AccelError):
+        op.run_strided(dX, dY, N, N - 1)
+    dX.close()
+    dY.close()
+
+
 @pytest.mark.parametrize("N", [17, 33, 50, 99, 127])
 def test_column_counts_of_upstreams_sweep_on_cfg2(gpu, N):
     """Upstream sweeps dim 16..128 in steps of 1 (main.cu:12): three quarters of those are
