@@ -265,11 +265,25 @@ def uniform_graph(n_rows, degree, n_cols, seed=0):
     return Graph(f"uniform:{n_rows}:{degree}:{n_cols}", indptr, indices, values, n_rows, n_cols)
 
 
+def columns_by_popularity(g):
+    """The same matrix with its columns renumbered by descending number of non-zeros (the
+    most referenced column becomes column 0): what a caller would get by ordering the rows
+    of X by popularity.  Columns inside a row are left in the order of the old numbering."""
+    count = np.bincount(g.indices, minlength=g.n_cols)
+    order = np.argsort(-count, kind="stable")                  # new id -> old id
+    new_of_old = np.empty(g.n_cols, dtype=np.int32)
+    new_of_old[order] = np.arange(g.n_cols, dtype=np.int32)
+    return Graph("bypopularity:" + g.name, g.indptr, new_of_old[g.indices], g.values, g.n_rows, g.n_cols)
+
+
 def workload(spec):
-    """cfg1..cfg5, fixture:<name>, local:<name>:<sigma> or uniform:<rows>:<degree>:<cols>."""
+    """cfg1..cfg5, fixture:<name>, local:<name>:<sigma>, uniform:<rows>:<degree>:<cols>, or
+    bypopularity:<any of these> for the same matrix with columns renumbered by popularity."""
     if spec in WORKLOADS:
         return WORKLOADS[spec]()
     kind, _, rest = spec.partition(":")
+    if kind == "bypopularity":
+        return columns_by_popularity(workload(rest))
     if kind == "fixture":
         return fixture_graph(rest)
     if kind == "local":

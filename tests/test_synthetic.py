@@ -144,3 +144,18 @@ def test_export_in_upstreams_layout(pkg, tmp_path):
     sip, six, _ = po.permute_csr(g.indptr, g.indices, g.values, perm)
     assert np.array_equal(ip, sip) and np.array_equal(ix, six)
     assert np.all(np.diff(np.diff(ip)) >= 0)
+
+
+def test_columns_by_popularity_is_the_same_matrix(pkg):
+    syn = pkg.synthetic
+    g = syn.cfg1()
+    p = syn.workload("bypopularity:cfg1")
+    count = np.bincount(p.indices, minlength=p.n_cols)
+    assert np.all(np.diff(count) <= 0)                     # column 0 is the most referenced
+    # the same product once X is permuted the same way
+    X = syn.dense_operand("cfg1", g.n_cols, 4)
+    old_count = np.bincount(g.indices, minlength=g.n_cols)
+    order = np.argsort(-old_count, kind="stable")
+    Y0 = so.csr(g.indptr, g.indices, g.values, g.n_cols) @ X
+    Y1 = so.csr(p.indptr, p.indices, p.values, p.n_cols) @ X[order]
+    assert np.allclose(Y0, Y1, rtol=1e-5, atol=1e-6)
