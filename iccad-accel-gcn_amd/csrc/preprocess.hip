@@ -155,6 +155,7 @@ struct Stats {
     int n_big_rows;     // rows with more than 32 times that
     int n_split_rows_alt, n_big_rows_alt;   // the same two for the alternative threshold
     int n_wide_rows;    // rows with more than kGroupWaveMax non-zeros
+    int hist[kDegBound + 1];   // rows of each degree 0..384 (what sizes the partition on the host)
     int sampled_nz;     // non-zeros looked at by locality_kernel
     int local_nz;       // ... whose column lies near their row
 };
@@ -171,6 +172,9 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
 {
     // grid-stride over rows; one set of atomics per workgroup
     __shared__ int part[kThreads / 64][11];
+    __shared__ int hist[kDegBound + 1];
+    for (int i = threadIdx.x; i <= kDegBound; i += kThreads) hist[i] = 0;
+    __syncthreads();
     int bad = 0, unsorted = 0, dmax = 0, zero = 0, lrow = 0, lblk = 0, srow = 0, brow = 0, srow2 = 0, brow2 = 0;
     int wrow = 0;
     for (int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x; r < rows;
@@ -192,6 +196,7 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
         srow2 += d > alt_split_deg;
         brow2 += d > 32 * alt_split_deg;
         wrow += d > kGroupWaveMax;
+        if (!row_bad && d <= kDegBound) atomicAdd(&hist[d], 1);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -232,6 +237,8 @@ __global__ __launch_bounds__(kThreads) void degree_kernel(const int32_t *__restr
         if (brow2) atomicAdd(&st->n_big_rows_alt, brow2);
         if (wrow) atomicAdd(&st->n_wide_rows, wrow);
     }
+    for (int i = threadIdx.x; i <= kDegBound; i += kThreads)      // after the barrier above: hist is complete
+        if (hist[i]) atomicAdd(&st->hist[i], hist[i]);
 }
 
 // Does the matrix have its non-zeros near the diagonal (of the rows x cols rectangle)?
@@ -746,9 +753,11 @@ __global__ __launch_bounds__(kThreads) void block_count_kernel(
 
 __global__ __launch_bounds__(kThreads) void emit_block4_kernel(
     const uint32_t *__restrict__ deg, const int32_t *__restrict__ s_indptr,
-    const int *__restrict__ run_start, const int *__restrict__ row_block, int64_t rows,
+    const int *__restrict__ run_start, const int *__restrict__ row_block, int64_t rows, int n_blocks,
     int4 *__restrict__ block4)
 {
+    // n_blocks = entries allocated; a row whose blocks would not fit writes nothing (the host
+    // compares the device's total with its own afterwards)
     const int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x;
     if (r >= rows) return;
     const int d = (int)deg[r];
@@ -757,6 +766,7 @@ __global__ __launch_bounds__(kThreads) void emit_block4_kernel(
     const int loc = s_indptr[r];
     if (d > kDegBound) {
         const int nseg = (d + kDegBound - 1) / kDegBound;
+        if (at + nseg > n_blocks) return;
         for (int k = 0; k < nseg; k++)
             block4[at + k] = make_int4(d, (int)r, loc + k * kDegBound,
                                        min(kDegBound, d - k * kDegBound));
@@ -767,7 +777,7 @@ __global__ __launch_bounds__(kThreads) void emit_block4_kernel(
     if (((int)r - run_start[r]) % rpb != 0) return;
     int n = 1;
     while (n < rpb && r + n < rows && (int)deg[r + n] == d) n++;
-    block4[at] = make_int4(d, (int)r, loc, (w << 16) + n);
+    if (at < n_blocks) block4[at] = make_int4(d, (int)r, loc, (w << 16) + n);
 }
 
 // ---------------------------------------------------------------------------
@@ -957,12 +967,41 @@ __device__ __forceinline__ int queue_of(int running_cost, const QueueCuts &qc)
     return q;
 }
 
+// The share boundaries, computed where the numbers are: queue q takes max(0, level - long_cost[q])
+// of the whole-row units' cost, level being the smallest common level that takes all of it.
+// One thread; total_cost points at the sum of the units' costs.
+__global__ void queue_cuts_kernel(const int *__restrict__ long_cost, const int *__restrict__ total_cost,
+                                  QueueCuts *__restrict__ out)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const long long short_cost = *total_cost;
+    long long lc[kXcds], lo = 0, hi = short_cost;
+    for (int q = 0; q < kXcds; q++) {
+        lc[q] = long_cost ? long_cost[q] : 0;
+        if (lc[q] + short_cost > hi) hi = lc[q] + short_cost;
+    }
+    while (lo < hi) {                                  // smallest level that takes all of it
+        const long long mid = (lo + hi) / 2;
+        long long taken = 0;
+        for (int q = 0; q < kXcds; q++) taken += mid > lc[q] ? mid - lc[q] : 0;
+        if (taken >= short_cost) hi = mid; else lo = mid + 1;
+    }
+    long long run = 0;
+    for (int q = 0; q < kXcds; q++) {
+        out->cut[q] = (int)(run < short_cost ? run : short_cost);
+        run += lo > lc[q] ? lo - lc[q] : 0;
+    }
+    out->cut[kXcds] = INT_MAX;
+}
+
 // first[q] = rank of the first unit of queue q (n for queues that get none); first must hold n on entry.
 __global__ __launch_bounds__(kThreads) void queue_first_kernel(const int *__restrict__ running, int n,
-                                                               QueueCuts qc, int *__restrict__ first)
+                                                               const QueueCuts *__restrict__ cuts,
+                                                               int *__restrict__ first)
 {
     const int sidx = blockIdx.x * kThreads + threadIdx.x;
     if (sidx >= n) return;
+    const QueueCuts qc = *cuts;
     const int q = queue_of(running[sidx], qc);
     const int q_prev = sidx == 0 ? -1 : queue_of(running[sidx - 1], qc);
     for (int i = q_prev + 1; i <= q; i++) first[i] = sidx;
@@ -977,11 +1016,12 @@ __global__ __launch_bounds__(kThreads) void queue_first_kernel(const int *__rest
 constexpr int kTailLight = 2048;             // two rounds of the 1,024 wavefronts a die holds
 __global__ __launch_bounds__(kThreads) void place_short_units_kernel(
     const int4 *__restrict__ units, const uint32_t *__restrict__ order, const int *__restrict__ running,
-    const int *__restrict__ heavy_before, int n, QueueCuts qc, const int *__restrict__ first,
-    PlanParams pp, int4 *__restrict__ work)
+    const int *__restrict__ heavy_before, int n, const QueueCuts *__restrict__ cuts,
+    const int *__restrict__ first, PlanParams pp, int4 *__restrict__ work)
 {
     const int sidx = blockIdx.x * kThreads + threadIdx.x;
     if (sidx >= n) return;
+    const QueueCuts qc = *cuts;
     const int q = queue_of(running[sidx], qc);
     const int f = first[q], n_q = first[q + 1] - f;
     const int h0 = heavy_before[f];
@@ -1007,8 +1047,12 @@ __global__ __launch_bounds__(kThreads) void place_short_units_kernel(
 static int partition_device(Arena *tmp, const uint32_t *deg, const int32_t *s_indptr, int64_t rows,
                             int32_t **block4_out, int64_t *n_blocks, hipStream_t s,
                             int64_t probe_row = -1, int64_t *blocks_before_probe = nullptr,
-                            int64_t *nnz_before_probe = nullptr)
+                            int64_t *nnz_before_probe = nullptr, int64_t known_blocks = -1,
+                            const int **total_blocks_dev = nullptr)
 {
+    // known_blocks >= 0: the host already knows the number of blocks (rows in ascending degree
+    // order: one run per degree, so the count follows from the degree histogram) and nothing
+    // is read back here; *total_blocks_dev then points at the device's own total for a later check
     DevBuf head(tmp), cnt(tmp), sums(tmp), rb(tmp), b4;
     int rc;
     if ((rc = head.alloc(sizeof(int) * (size_t)rows))) return rc;
@@ -1024,18 +1068,21 @@ static int partition_device(Arena *tmp, const uint32_t *deg, const int32_t *s_in
     if ((rc = device_scan<SumOp, false>(cnt.as<int>(), rows, rb.as<int>(), rb.as<int>() + rows,
                                         sums.as<int>(), s)))
         return rc;
-    int nb = 0, before = 0, nnz_before = 0;
-    ACCEL_HIP(hipMemcpyAsync(&nb, rb.as<int>() + rows, sizeof(int), hipMemcpyDeviceToHost, s));
-    if (blocks_before_probe && probe_row >= 0 && probe_row <= rows)   // rb[rows] is the total
-        ACCEL_HIP(hipMemcpyAsync(&before, rb.as<int>() + probe_row, sizeof(int), hipMemcpyDeviceToHost, s));
-    if (nnz_before_probe && probe_row >= 0 && probe_row <= rows)
-        ACCEL_HIP(hipMemcpyAsync(&nnz_before, s_indptr + probe_row, sizeof(int), hipMemcpyDeviceToHost, s));
-    ACCEL_HIP(hipStreamSynchronize(s));
-    if (blocks_before_probe) *blocks_before_probe = before;
-    if (nnz_before_probe) *nnz_before_probe = nnz_before;
+    int nb = (int)known_blocks, before = 0, nnz_before = 0;
+    if (known_blocks < 0) {
+        ACCEL_HIP(hipMemcpyAsync(&nb, rb.as<int>() + rows, sizeof(int), hipMemcpyDeviceToHost, s));
+        if (blocks_before_probe && probe_row >= 0 && probe_row <= rows)   // rb[rows] is the total
+            ACCEL_HIP(hipMemcpyAsync(&before, rb.as<int>() + probe_row, sizeof(int), hipMemcpyDeviceToHost, s));
+        if (nnz_before_probe && probe_row >= 0 && probe_row <= rows)
+            ACCEL_HIP(hipMemcpyAsync(&nnz_before, s_indptr + probe_row, sizeof(int), hipMemcpyDeviceToHost, s));
+        ACCEL_HIP(hipStreamSynchronize(s));
+        if (blocks_before_probe) *blocks_before_probe = before;
+        if (nnz_before_probe) *nnz_before_probe = nnz_before;
+    }
+    if (total_blocks_dev) *total_blocks_dev = rb.as<int>() + rows;
     if ((rc = b4.alloc(sizeof(int4) * (size_t)nb))) return rc;
     emit_block4_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(
-        deg, s_indptr, head.as<int>(), rb.as<int>(), rows, b4.as<int4>());
+        deg, s_indptr, head.as<int>(), rb.as<int>(), rows, nb, b4.as<int4>());
     ACCEL_HIP(hipGetLastError());
     *n_blocks = nb;
     *block4_out = static_cast<int32_t *>(b4.release());
@@ -1091,10 +1138,11 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
 // row ids have neighbouring columns (most graphs with a meaningful vertex order)
 // lose that locality to the degree sort; this gives it back: at any time a die
 // works on a narrow band of the caller's rows.
-// The host sees 121 bin totals, eight queue loads, one unit count, one total cost
-// and nine share boundaries, to size the queues.
+// The host sees 121 bin totals and nine share boundaries, in one synchronisation, to size
+// the queues (plus the number of whole-row units when entries are cut into smaller units).
 static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const int32_t *s_indptr,
-                           int64_t first_long, int64_t n_short, const uint32_t *perm, hipStream_t s)
+                           int64_t first_long, int64_t n_short, const uint32_t *perm,
+                           const int *total_blocks_dev, hipStream_t s)
 {
     // "long" here = rows cut into pieces (more than plan_split non-zeros); n_short = block4
     // entries of all other rows (they precede the rest in block4)
@@ -1105,7 +1153,6 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         lrank(tmp);
     int rc;
     int tot[kPlanBins + 1] = {0};
-    int long_cost[kXcds] = {0};
     // the order by row id is kept to 16 bits (two passes of the sort): bands of rows, not single
     // rows, are what the caches see; equal keys stay in row order (the sort is stable)
     int key_shift = 0;
@@ -1148,7 +1195,6 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         plan_totals_kernel<<<dim3(1), dim3(128), 0, s>>>(grp_units.as<int>(), (int)n_long,
                                                        totals.as<int>());
         ACCEL_HIP(hipMemcpyAsync(tot, totals.p, sizeof(tot), hipMemcpyDeviceToHost, s));
-        ACCEL_HIP(hipMemcpyAsync(long_cost, qload.p, sizeof(long_cost), hipMemcpyDeviceToHost, s));
     } else {
         ACCEL_HIP(hipMemsetAsync(dslot.p, 0, sizeof(int), s));
     }
@@ -1163,33 +1209,23 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         if ((rc = device_scan<SumOp, false>(scnt.as<int>(), n_short, scnt.as<int>(),
                                             scnt.as<int>() + n_short, ssums.as<int>(), s)))
             return rc;
-        ACCEL_HIP(hipMemcpyAsync(&n_short_units32, scnt.as<int>() + n_short, sizeof(int),
-                                 hipMemcpyDeviceToHost, s));
+        // with units of a whole block4 entry (large matrices) there is one unit per entry and
+        // nothing to wait for; smaller units are counted on the device
+        n_short_units32 = (int)n_short;
+        if (unit_nz < kDegBound) {
+            ACCEL_HIP(hipMemcpyAsync(&n_short_units32, scnt.as<int>() + n_short, sizeof(int),
+                                     hipMemcpyDeviceToHost, s));
+            ACCEL_HIP(hipStreamSynchronize(s));
+        }
     }
-    ACCEL_HIP(hipStreamSynchronize(s));
     const int64_t n_short_units = n_short_units32;
-    PlanParams pp;
-    BinOffsets bo;
-    for (int q = 0; q < kXcds; q++) pp.queue_long[q] = 0;
-    for (int b = 0; b < kPlanBins; b++) bo.off[b] = 0;
-    if (n_long > 0)
-        // a die first takes the pieces of the rows with the most groups (the longest
-        // rows), one group after the other, then those of the next class, ...
-        for (int ng = kMaxGroups; ng >= kXcds; ng /= 2)
-            for (int g = 0; g < ng; g++) {
-                const int b = plan_bin(ng, g);
-                bo.off[b] = pp.queue_long[g % kXcds];
-                pp.queue_long[g % kXcds] += tot[b + 1] - tot[b];
-            }
-    const int64_t n_long_units = n_long > 0 ? tot[kPlanBins] : 0;
 
     // whole-row units: list them, order them by the caller's row id, cut the sequence into
     // one share per queue so that long pieces + share cost about the same everywhere
-    DevBuf units(tmp), key(tmp), cost(tmp), heavy(tmp), csums(tmp), first(tmp);
+    DevBuf units(tmp), key(tmp), cost(tmp), heavy(tmp), csums(tmp), first(tmp), cuts(tmp);
     uint32_t *order = nullptr;
-    QueueCuts qc;
     int first_h[kXcds + 1];
-    for (int q = 0; q <= kXcds; q++) { qc.cut[q] = 0; first_h[q] = 0; }
+    for (int q = 0; q <= kXcds; q++) first_h[q] = 0;
     if (n_short_units > 0) {
         const int n = (int)n_short_units;
         uint32_t *sorted_key = nullptr;
@@ -1199,6 +1235,7 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         if ((rc = heavy.alloc(sizeof(int) * (size_t)(n + 1)))) return rc;
         if ((rc = csums.alloc(sizeof(int) * (size_t)(n / kTile + 4)))) return rc;
         if ((rc = first.alloc(sizeof(int) * (kXcds + 1)))) return rc;
+        if ((rc = cuts.alloc(sizeof(QueueCuts)))) return rc;
         list_short_units_kernel<<<dim3(grid_for(n_short)), dim3(kThreads), 0, s>>>(
             reinterpret_cast<const int4 *>(h->block4), (int)n_short, unit_nz, scnt.as<int>(), perm,
             key_shift, units.as<int4>(), key.as<uint32_t>());
@@ -1213,33 +1250,38 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         if ((rc = device_scan<SumOp, false>(heavy.as<int>(), n, heavy.as<int>(), heavy.as<int>() + n,
                                             csums.as<int>(), s)))
             return rc;
-        int short_cost = 0;
-        ACCEL_HIP(hipMemcpyAsync(&short_cost, cost.as<int>() + n, sizeof(int), hipMemcpyDeviceToHost, s));
-        ACCEL_HIP(hipStreamSynchronize(s));
-        // raise a common level: queue q takes max(0, level - long_cost[q]) of the short cost
-        int64_t lo = 0, hi = (int64_t)short_cost;
-        for (int q = 0; q < kXcds; q++) hi = std::max<int64_t>(hi, (int64_t)long_cost[q] + short_cost);
-        auto taken = [&](int64_t level) {
-            int64_t t = 0;
-            for (int q = 0; q < kXcds; q++) t += std::max<int64_t>(0, level - long_cost[q]);
-            return t;
-        };
-        while (lo < hi) {                              // smallest level that takes all of it
-            const int64_t mid = (lo + hi) / 2;
-            if (taken(mid) >= short_cost) hi = mid; else lo = mid + 1;
-        }
-        int64_t run = 0;
-        for (int q = 0; q < kXcds; q++) {
-            qc.cut[q] = (int)std::min<int64_t>(run, short_cost);
-            run += std::max<int64_t>(0, lo - long_cost[q]);
-        }
-        qc.cut[kXcds] = INT_MAX;
+        queue_cuts_kernel<<<dim3(1), dim3(1), 0, s>>>(n_long > 0 ? qload.as<int>() : nullptr, cost.as<int>() + n,
+                                                      cuts.as<QueueCuts>());
         if ((rc = fill_u32(first.p, (uint32_t)n, kXcds + 1, s))) return rc;
-        queue_first_kernel<<<dim3(grid_for(n)), dim3(kThreads), 0, s>>>(cost.as<int>(), n, qc,
+        queue_first_kernel<<<dim3(grid_for(n)), dim3(kThreads), 0, s>>>(cost.as<int>(), n, cuts.as<QueueCuts>(),
                                                                        first.as<int>());
         ACCEL_HIP(hipMemcpyAsync(first_h, first.p, sizeof(first_h), hipMemcpyDeviceToHost, s));
-        ACCEL_HIP(hipStreamSynchronize(s));
     }
+    // the one synchronisation of the plan: bin totals, share boundaries, and the device's own
+    // count of block4 entries (the host sized them from the degree histogram)
+    int device_blocks = (int)h->n_blocks;
+    if (total_blocks_dev)
+        ACCEL_HIP(hipMemcpyAsync(&device_blocks, total_blocks_dev, sizeof(int), hipMemcpyDeviceToHost, s));
+    ACCEL_HIP(hipStreamSynchronize(s));
+    if (device_blocks != (int)h->n_blocks) {
+        set_error("internal: the partition has %d blocks, %lld were expected from the degree histogram",
+                  device_blocks, (long long)h->n_blocks);
+        return ACCEL_ERR_STATE;
+    }
+    PlanParams pp;
+    BinOffsets bo;
+    for (int q = 0; q < kXcds; q++) pp.queue_long[q] = 0;
+    for (int b = 0; b < kPlanBins; b++) bo.off[b] = 0;
+    if (n_long > 0)
+        // a die first takes the pieces of the rows with the most groups (the longest
+        // rows), one group after the other, then those of the next class, ...
+        for (int ng = kMaxGroups; ng >= kXcds; ng /= 2)
+            for (int g = 0; g < ng; g++) {
+                const int b = plan_bin(ng, g);
+                bo.off[b] = pp.queue_long[g % kXcds];
+                pp.queue_long[g % kXcds] += tot[b + 1] - tot[b];
+            }
+    const int64_t n_long_units = n_long > 0 ? tot[kPlanBins] : 0;
     int64_t per_queue = 0;
     for (int q = 0; q < kXcds; q++)
         per_queue = std::max<int64_t>(per_queue, (int64_t)pp.queue_long[q] + (first_h[q + 1] - first_h[q]));
@@ -1258,7 +1300,7 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
             piece_nz, lrank.as<int>(), bo, dwork.as<int4>());
     if (n_short_units > 0)
         place_short_units_kernel<<<dim3(grid_for(n_short_units)), dim3(kThreads), 0, s>>>(
-            units.as<int4>(), order, cost.as<int>(), heavy.as<int>(), (int)n_short_units, qc,
+            units.as<int4>(), order, cost.as<int>(), heavy.as<int>(), (int)n_short_units, cuts.as<QueueCuts>(),
             first.as<int>(), pp, dwork.as<int4>());
     ACCEL_HIP(hipGetLastError());
     ACCEL_HIP(hipStreamSynchronize(s));
@@ -1514,12 +1556,25 @@ int preprocess_device(accel_handle *h)
     // ---- partition ----------------------------------------------------------
     // (before the sorted CSR: its one synchronisation also tells how many non-zeros the rows
     // that are not split hold, which sizes the gather below)
+    // Sizes from the degree histogram: the rows are in ascending degree order, so every degree
+    // d <= 384 forms one run, cut into ceil(count / rows per block) blocks.
     int32_t *b4 = nullptr;
-    int64_t nb = 0;
+    int64_t nb = hs.n_long_blocks;
     int64_t n_short_entries = 0;   // block4 entries of the rows that are not cut into pieces
     int64_t nnz_short = 0;         // their non-zeros
-    if ((rc = partition_device(&tmp, sdeg, sip.as<int32_t>(), rows, &b4, &nb, s, first_long, &n_short_entries,
-                               &nnz_short)))
+    for (int d = 1; d <= kDegBound; d++) {
+        int w, rpb;
+        slice_rule(d, w, rpb);
+        const int64_t blocks = ((int64_t)hs.hist[d] + rpb - 1) / rpb;
+        nb += blocks;
+        if (d <= h->plan_split) {
+            n_short_entries += blocks;
+            nnz_short += (int64_t)d * hs.hist[d];
+        }
+    }
+    const int *total_blocks_dev = nullptr;
+    if ((rc = partition_device(&tmp, sdeg, sip.as<int32_t>(), rows, &b4, &nb, s, -1, nullptr, nullptr, nb,
+                               &total_blocks_dev)))
         return rc;
     h->block4 = b4;
     h->n_blocks = nb;
@@ -1562,7 +1617,8 @@ int preprocess_device(accel_handle *h)
     }
 
     // ---- work list ------------------------------------------------------------
-    if ((rc = build_work_list(&tmp, h, gcount.as<int>(), sip.as<int32_t>(), first_long, n_short_entries, perm, s)))
+    if ((rc = build_work_list(&tmp, h, gcount.as<int>(), sip.as<int32_t>(), first_long, n_short_entries, perm,
+                              total_blocks_dev, s)))
         return rc;
 
     h->slab = slab.release();
