@@ -388,11 +388,15 @@ def main():
         base, n_rows, Yc = cpu_baseline(g, X, N)
         result["cpu_baseline"] = base
         # parity of the timed output on the baseline's rows (fp64 reference, scaled error)
-        from oracle import spmm_oracle as so
+        from oracle import c_oracle, spmm_oracle as so
         Y = dY.to_numpy(np.float32, (g.n_rows, N))[:n_rows]
-        nz = int(g.indptr[n_rows])
-        R, S = so.spmm_fp64(g.indptr[: n_rows + 1], g.indices[:nz], g.values[:nz], X)
-        err = so.scaled_error(Y, R, S)
+        threads = min(16, os.cpu_count() or 1)          # the checker may use the host's cores; the baseline above does not
+        err, slab = 0.0, max(1, (64 << 20) // N)        # 512 MB of fp64 reference at a time
+        for r0 in range(0, n_rows, slab):
+            r1 = min(n_rows, r0 + slab)
+            R, S = c_oracle.spmm_csr_f64(g.indptr[r0:r1 + 1], g.indices, g.values, X, threads=threads)
+            err = max(err, so.scaled_error(Y[r0:r1], R, S))
+            del R, S
         result["parity"] = {"rows_checked": n_rows, "scaled_error": err, "tolerance": so.TOL,
                             "ok": bool(err <= so.TOL)}
         if err > so.TOL:
