@@ -16,6 +16,7 @@
 #include <chrono>
 #include <cstdio>
 #include <memory>
+#include <new>
 #include <vector>
 
 #include "internal.h"
@@ -152,18 +153,36 @@ int accel_save_state(const accel_handle *h, const char *path)
         out.f = fopen(tmp.c_str(), "wb");
         if (!out.f) { set_error("cannot create %s", tmp.c_str()); return ACCEL_ERR_IO; }
         bool ok = fwrite(&hd, sizeof hd, 1, out.f) == 1;
+        int rc = ACCEL_OK;
         std::vector<uint32_t> host;
-        for (int i = 0; i < kNumArrays && ok; i++) {
+        for (int i = 0; i < kNumArrays && ok && !rc; i++) {
             if (hd.words[i] == 0) continue;
-            host.resize((size_t)hd.words[i]);
-            ACCEL_HIP(hipMemcpy(host.data(), arrays[i], sizeof(uint32_t) * host.size(), hipMemcpyDeviceToHost));
+            try {
+                host.resize((size_t)hd.words[i]);
+            } catch (const std::bad_alloc &) {
+                set_error("host allocation of %lld bytes failed", (long long)hd.words[i] * 4);
+                rc = ACCEL_ERR_ALLOC;
+                break;
+            }
+            const hipError_t e =
+                hipMemcpy(host.data(), arrays[i], sizeof(uint32_t) * host.size(), hipMemcpyDeviceToHost);
+            if (e != hipSuccess) {
+                set_error("download of the state failed: %s", hipGetErrorString(e));
+                rc = ACCEL_ERR_HIP;
+                break;
+            }
             ok = fwrite(host.data(), sizeof(uint32_t), host.size(), out.f) == host.size();
         }
         ok = ok && fflush(out.f) == 0;
-        if (!ok) {
+        if (!rc && !ok) {
             set_error("write to %s failed", tmp.c_str());
+            rc = ACCEL_ERR_IO;
+        }
+        if (rc) {
+            fclose(out.f);
+            out.f = nullptr;
             (void)remove(tmp.c_str());
-            return ACCEL_ERR_IO;
+            return rc;
         }
     }
     if (rename(tmp.c_str(), path) != 0) {
@@ -213,6 +232,20 @@ int accel_load_state(accel_handle *h, const char *path)
                  hd.plan_groups == 64);
     for (int i = 0; i < kNumArrays && sane; i++) sane = hd.words[i] == want[i];
     if (!sane) { set_error("%s: inconsistent header", path); return ACCEL_ERR_META; }
+    // the file must be exactly as long as the header says, before anything is allocated from it
+    {
+        int64_t expect = (int64_t)sizeof(StateHeader);
+        for (int i = 0; i < kNumArrays; i++) expect += 4 * hd.words[i];
+        const long at = ftell(in.f);
+        if (at < 0 || fseek(in.f, 0, SEEK_END) != 0) { set_error("%s: cannot seek", path); return ACCEL_ERR_IO; }
+        const long len = ftell(in.f);
+        if (fseek(in.f, at, SEEK_SET) != 0) { set_error("%s: cannot seek", path); return ACCEL_ERR_IO; }
+        if ((int64_t)len != expect) {
+            set_error("%s: %lld bytes, the header describes %lld (truncated or damaged file)", path,
+                      (long long)len, (long long)expect);
+            return ACCEL_ERR_IO;
+        }
+    }
 
     release_products(h);
     if (h->rows == 0) {
@@ -237,7 +270,12 @@ int accel_load_state(accel_handle *h, const char *path)
     std::vector<uint32_t> host;
     for (int i = 0; i < kNumArrays; i++) {
         if (hd.words[i] == 0) continue;
-        host.resize((size_t)hd.words[i]);
+        try {
+            host.resize((size_t)hd.words[i]);
+        } catch (const std::bad_alloc &) {
+            set_error("host allocation of %lld bytes failed", (long long)hd.words[i] * 4);
+            return fail(ACCEL_ERR_ALLOC);
+        }
         if (fread(host.data(), sizeof(uint32_t), host.size(), in.f) != host.size()) {
             set_error("%s: truncated", path);
             return fail(ACCEL_ERR_IO);

@@ -126,6 +126,7 @@ def test_damaged_truncated_and_missing_files(gpu, tmp_path):
     refused(flipped, gpu._lib.ERR_META)
     refused(raw[: len(raw) - 100], gpu._lib.ERR_IO)      # truncated payload
     refused(raw[:50], gpu._lib.ERR_IO)                   # truncated header
+    refused(raw + b"\0" * 8, gpu._lib.ERR_IO)            # longer than its header says
     refused(b"not a state file" * 40, gpu._lib.ERR_META)
     with pytest.raises(gpu.AccelError) as e:
         b.load_state(tmp_path / "nothing_here.accelstate")
