@@ -281,6 +281,14 @@ def main():
         from_cache_ms = op2.info.preprocess_ms
         op2.close()
     log(f"[bench] preprocess from a saved state ({state_mb:.1f} MB): {from_cache_ms:.1f} ms")
+    # new values on the same structure (accel_update_values), from an array already on the device
+    dV = pkg.DeviceBuffer.from_numpy(np.ascontiguousarray(g.values, dtype=np.float32))
+    op.update_values(dV)
+    t0 = time.perf_counter()
+    op.update_values(dV)
+    update_values_ms = (time.perf_counter() - t0) * 1e3
+    dV.close()
+    log(f"[bench] values replaced on the same structure: {update_values_ms:.2f} ms")
     dX = pkg.DeviceBuffer.from_numpy(X)
     dY = pkg.DeviceBuffer(g.n_rows * N * 4)
     dY.fill_u32(0x7FC00000)
@@ -346,6 +354,7 @@ def main():
                    "preprocess_ms": round(info.preprocess_ms, 2),
                    "preprocess_first_call_ms": round(first_preprocess_ms, 2),
                    "preprocess_from_cache_ms": round(from_cache_ms, 2),
+                   "update_values_ms": round(update_values_ms, 2),
                    "reference_protocol_ms": round(ref_protocol_ms, 5),
                    "plan": {"split_nz": int(info.plan_split_nz), "groups": int(info.plan_groups),
                             "unit_nz": int(info.plan_unit_nz), "panel": a.panel}},

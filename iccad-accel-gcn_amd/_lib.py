@@ -74,6 +74,7 @@ SIGNATURES = {
     "accel_set_plan_panel": (C.c_int, [vp, C.c_int]),
     "accel_save_state": (C.c_int, [vp, C.c_char_p]),
     "accel_load_state": (C.c_int, [vp, C.c_char_p]),
+    "accel_update_values": (C.c_int, [vp, vp, C.c_int]),
     "accel_check_block4": (C.c_int, [vp, i32p, C.c_int64]),
     "accel_get_info": (C.c_int, [vp, C.POINTER(Info)]),
     "accel_get_block4": (C.c_int, [vp, i32p, C.c_int64]),

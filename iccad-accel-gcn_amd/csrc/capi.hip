@@ -475,6 +475,37 @@ int accel_preprocess(accel_handle *h)
     return rc;
 }
 
+int accel_update_values(accel_handle *h, const float *val, int flags)
+{
+    clear_error();
+    if (!h) { set_error("accel_update_values: null handle"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_update_values: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (flags != ACCEL_PTR_HOST && flags != ACCEL_PTR_DEVICE) {
+        set_error("accel_update_values: unknown flags %d", flags);
+        return ACCEL_ERR_ARG;
+    }
+    if (h->nnz == 0) return ACCEL_OK;
+    if (!val) { set_error("accel_update_values: null array"); return ACCEL_ERR_ARG; }
+    const size_t bytes = sizeof(float) * (size_t)h->nnz;
+    if (flags == ACCEL_PTR_DEVICE)
+        if (int rc = check_operand(h, val, bytes, "accel_update_values", "val")) return rc;
+    if (!h->owns_input && flags != ACCEL_PTR_DEVICE) {
+        set_error("accel_update_values: this handle borrows its CSR from device memory; pass the new "
+                  "values as a device array (ACCEL_PTR_DEVICE)");
+        return ACCEL_ERR_ARG;
+    }
+    // runs of this handle that are still in flight read the arrays rewritten below
+    ACCEL_HIP(hipDeviceSynchronize());
+    if (h->owns_input) {
+        if (val != h->val)
+            ACCEL_HIP(hipMemcpy(const_cast<float *>(h->val), val, bytes,
+                                flags == ACCEL_PTR_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice));
+    } else {
+        h->val = val;                       // borrowed from now on (it may be the same array, rewritten)
+    }
+    return refresh_sorted_csr(h, nullptr);
+}
+
 int accel_get_info(const accel_handle *h, accel_info *out)
 {
     clear_error();

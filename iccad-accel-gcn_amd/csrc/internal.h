@@ -108,6 +108,7 @@ struct accel_handle {
     bool local = false;               // most non-zeros lie near the diagonal (sampled)
     int64_t n_split_rows = 0;         // rows with more than plan_split non-zeros
     int64_t n_big_rows = 0;           // of those, rows with more than 32 * plan_split
+    int64_t nnz_short = 0;            // non-zeros of the rows that are not split
     int64_t n_wide_rows = 0;          // rows with more than 1,024 non-zeros (regrouped by a workgroup each)
     int64_t n_blocks = 0, n_long_blocks = 0, n_long_rows = 0, n_zero_rows = 0;
     int32_t max_degree = 0;
@@ -128,6 +129,7 @@ namespace accel {
 // preprocess.hip
 int preprocess_device(accel_handle *h);
 int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s);
+int refresh_sorted_csr(accel_handle *h, hipStream_t s);
 int hash_words_device(const void *words_dev, int64_t n, uint64_t seed, uint64_t *out_dev, hipStream_t s);
 // capi.hip
 void release_products(accel_handle *h);

@@ -1399,44 +1399,57 @@ int hash_words_device(const void *words_dev, int64_t n, uint64_t seed, uint64_t 
     return ACCEL_OK;
 }
 
-// The degree-sorted copy of the CSR from the caller's arrays, perm, s_indptr and the
-// plan's split threshold: what accel_preprocess builds between the sort and the
-// partition.  Used when those products come from a saved state.  Needs h->perm (or
-// identity_perm), h->s_indptr, h->n_split_rows and h->plan_groups; sets s_idx, s_val,
-// owns_sorted.  nnz_short = non-zeros of the rows that are not split.
-int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s)
+// The non-zeros of the caller's CSR gathered into the degree-sorted copy the handle owns
+// (s_idx, s_val), in place: rows that stay whole keep the order of their non-zeros, split rows
+// are regrouped by column group.  Needs perm (or identity_perm), s_indptr, nnz_short,
+// n_split_rows, n_wide_rows and plan_groups.  This is also how new values on an unchanged
+// structure reach the copy the kernels read.
+int refresh_sorted_csr(accel_handle *h, hipStream_t s)
 {
-    const int64_t rows = h->rows, nnz = h->nnz, n_long = h->n_split_rows, first_long = rows - n_long;
-    if (h->identity_perm && n_long == 0) {
+    if (!h->owns_sorted) {                  // the sorted copy is the caller's CSR itself
         h->s_idx = h->idx;
         h->s_val = h->val;
-        h->owns_sorted = false;
         return ACCEL_OK;
     }
-    DevBuf sidx, sval, tiles;
-    int rc;
-    if ((rc = sidx.alloc(sizeof(int32_t) * (size_t)nnz))) return rc;
-    if ((rc = sval.alloc(sizeof(float) * (size_t)nnz))) return rc;
+    const int64_t rows = h->rows, n_long = h->n_split_rows, first_long = rows - n_long;
+    const int64_t nnz_short = h->nnz_short;
+    int32_t *sidx = const_cast<int32_t *>(h->s_idx);
+    float *sval = const_cast<float *>(h->s_val);
+    DevBuf tiles;
     if (nnz_short > 0) {
         if (h->identity_perm) {
-            ACCEL_HIP(hipMemcpyAsync(sidx.p, h->idx, sizeof(int32_t) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
-            ACCEL_HIP(hipMemcpyAsync(sval.p, h->val, sizeof(float) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
+            ACCEL_HIP(hipMemcpyAsync(sidx, h->idx, sizeof(int32_t) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
+            ACCEL_HIP(hipMemcpyAsync(sval, h->val, sizeof(float) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
         } else {
-            if ((rc = tiles.alloc(sizeof(int) * (size_t)(nnz_short / kPermuteTile + 2)))) return rc;
+            if (int rc = tiles.alloc(sizeof(int) * (size_t)(nnz_short / kPermuteTile + 2))) return rc;
             launch_permute_csr(h->indptr, h->idx, h->val, h->perm, h->s_indptr, rows, first_long, nnz_short,
-                               tiles.as<int>(), sidx.as<int32_t>(), sval.as<float>(), s);
+                               tiles.as<int>(), sidx, sval, s);
         }
     }
     if (n_long > 0)
         launch_group_long_rows(h->indptr, h->idx, h->val, h->perm, h->s_indptr, first_long, n_long,
-                               std::min<int64_t>(h->n_wide_rows, n_long), h->plan_groups,
-                               sidx.as<int32_t>(), sval.as<float>(), nullptr, s);
+                               std::min<int64_t>(h->n_wide_rows, n_long), h->plan_groups, sidx, sval, nullptr, s);
     ACCEL_HIP(hipGetLastError());
-    ACCEL_HIP(hipStreamSynchronize(s));
-    h->s_idx = static_cast<int32_t *>(sidx.release());
-    h->s_val = static_cast<float *>(sval.release());
-    h->owns_sorted = true;
+    ACCEL_HIP(hipStreamSynchronize(s));     // `tiles` is released on return
     return ACCEL_OK;
+}
+
+// The degree-sorted copy of the CSR for products that come from a saved state (perm,
+// s_indptr, the plan): allocates it and fills it as above.  nnz_short = non-zeros of the
+// rows that are not split.
+int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s)
+{
+    h->nnz_short = nnz_short;
+    h->owns_sorted = !(h->identity_perm && h->n_split_rows == 0);
+    if (h->owns_sorted) {
+        DevBuf sidx, sval;
+        int rc;
+        if ((rc = sidx.alloc(sizeof(int32_t) * (size_t)h->nnz))) { h->owns_sorted = false; return rc; }
+        if ((rc = sval.alloc(sizeof(float) * (size_t)h->nnz))) { h->owns_sorted = false; return rc; }
+        h->s_idx = static_cast<int32_t *>(sidx.release());
+        h->s_val = static_cast<float *>(sval.release());
+    }
+    return refresh_sorted_csr(h, s);        // on failure release_products frees what was allocated
 }
 
 int preprocess_device(accel_handle *h)
@@ -1622,6 +1635,7 @@ int preprocess_device(accel_handle *h)
         return rc;
 
     h->slab = slab.release();
+    h->nnz_short = nnz_short;
     h->s_indptr = sip.as<int32_t>();
     h->perm = permbuf.as<int32_t>();                 // null for sorted input
     if (!own_copy) {

@@ -686,8 +686,8 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     int panel = N;
     const int want = h->plan_panel_option > 0 ? h->plan_panel_option : kPanel;
     const bool forced = h->plan_panel_option > 0;
-    if (mode == 0 && N > want && N % want == 0 &&
-        (forced || (h->nnz >= kPanelMinNnz && h->nnz >= 16 * h->rows)))
+    if (mode == 0 && N > want &&
+        (forced || (N % want == 0 && h->nnz >= kPanelMinNnz && h->nnz >= 16 * h->rows)))
         panel = want;
     // operands below 4 GiB are addressed with 32-bit byte offsets (see gather_row)
     const bool wide = (uint64_t)h->cols * (uint64_t)ld * 4u > 0xFFFFFFFFull;

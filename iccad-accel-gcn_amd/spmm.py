@@ -95,6 +95,23 @@ class AccelSpMM:
         self._info = info
         return self
 
+    def update_values(self, values) -> "AccelSpMM":
+        """New values for the same structure (see accel_update_values): a numpy array of nnz
+        floats in the CSR's order, or, for device-resident values, an object with
+        ``data_ptr()`` / a raw address (required when the CSR was given with ``device=True``;
+        the operator then borrows that array)."""
+        self.info
+        if isinstance(values, np.ndarray):
+            v = _lib.as_f32(values)
+            if v.size != self.nnz:
+                raise AccelError(_lib.ERR_ARG, f"values has {v.size} entries, the CSR has {self.nnz} non-zeros")
+            check(lib().accel_update_values(self._h, ptr(v), _lib.PTR_HOST))
+        else:
+            check(lib().accel_update_values(self._h, _lib.dev_ptr(values, self.nnz * 4, "values"), _lib.PTR_DEVICE))
+            if self._keep is not None and len(self._keep) == 3:
+                self._keep = (self._keep[0], self._keep[1], values)
+        return self
+
     def set_panel(self, columns: int) -> None:
         """Column-panel width of the following runs (0: automatic; see accel_set_plan_panel)."""
         check(lib().accel_set_plan_panel(self._h, int(columns)))

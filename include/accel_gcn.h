@@ -149,12 +149,27 @@ int accel_set_plan_team(accel_handle *h, int mode);
 int accel_save_state(const accel_handle *h, const char *path);
 int accel_load_state(accel_handle *h, const char *path);
 
+/* New values for the non-zeros of an unchanged structure (indptr and idx as they were
+ * at accel_create), e.g. edge weights that change between training steps.  Upstream's
+ * kernel reads the caller's `val` on every launch (spmm_accel.cu:75), so a caller that
+ * rewrites the array sees the new weights at once; this library computes from its
+ * degree-sorted copy, which this call refreshes (one gather pass over the non-zeros,
+ * about half the time of accel_preprocess; sort, metadata and launch plan are kept).
+ * val: nnz floats in the order of the CSR given to accel_create; flags says where it
+ * lives (ACCEL_PTR_HOST or ACCEL_PTR_DEVICE).  A handle that uploaded its CSR copies
+ * the values into its own array; a handle that borrows device arrays needs a device
+ * array and borrows that one from now on (it may be the same array, rewritten in
+ * place).  Synchronous, and it waits for all work on the device first: do not call it
+ * while a stream is capturing.  A saved state holds no values and stays valid. */
+int accel_update_values(accel_handle *h, const float *val, int flags);
+
 /* Column panels (no counterpart upstream, which always walks all N columns of a row
- * at once, spmm_accel.cu:37-48): when N is a multiple of `columns` and larger, one
- * accel_run computes Y one panel of `columns` columns at a time, all work units for
- * the first panel before the next, so that the caches only have to hold that slice
- * of X.  0 (the default) lets the library choose from N and the size of the matrix.
- * Takes effect at the next accel_run; needs 16-byte aligned X and Y. */
+ * at once, spmm_accel.cu:37-48): one accel_run computes Y one panel of `columns`
+ * columns at a time (the last one narrower when N is not a multiple), all work units
+ * for the first panel before the next, so that the caches only have to hold that slice
+ * of X.  0 (the default) lets the library choose from N and the size of the matrix
+ * (panels of 64 for N = 128, 192, ... on large matrices).
+ * Takes effect at the next accel_run; needs N % 4 == 0 and 16-byte aligned X and Y. */
 int accel_set_plan_panel(accel_handle *h, int columns);
 
 /* Check externally produced metadata (a .block4 file) against what

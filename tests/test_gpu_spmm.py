@@ -107,7 +107,8 @@ def test_column_counts_of_upstreams_sweep_on_cfg2(gpu, N):
     op.close()
 
 
-@pytest.mark.parametrize("N,panel", [(64, 32), (128, 32), (128, 64), (96, 32), (48, 16), (256, 128)])
+@pytest.mark.parametrize("N,panel", [(64, 32), (128, 32), (128, 64), (96, 32), (48, 16), (256, 128),
+                                     (100, 64), (100, 32), (72, 20), (8, 4)])    # the last panel narrower
 def test_forced_column_panels(gpu, mixed, N, panel):
     """A run cut into column panels computes the same product (a narrower panel gives a row
     more lane groups, so the order of the additions may differ)."""
