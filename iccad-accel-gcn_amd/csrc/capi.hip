@@ -503,7 +503,7 @@ int accel_update_values(accel_handle *h, const float *val, int flags)
     } else {
         h->val = val;                       // borrowed from now on (it may be the same array, rewritten)
     }
-    return refresh_sorted_csr(h, nullptr);
+    return refresh_sorted_csr(h, true, nullptr);
 }
 
 int accel_get_info(const accel_handle *h, accel_info *out)

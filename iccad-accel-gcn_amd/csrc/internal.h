@@ -129,7 +129,7 @@ namespace accel {
 // preprocess.hip
 int preprocess_device(accel_handle *h);
 int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s);
-int refresh_sorted_csr(accel_handle *h, hipStream_t s);
+int refresh_sorted_csr(accel_handle *h, bool values_only, hipStream_t s);
 int hash_words_device(const void *words_dev, int64_t n, uint64_t seed, uint64_t *out_dev, hipStream_t s);
 // capi.hip
 void release_products(accel_handle *h);

@@ -533,7 +533,7 @@ __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
             if ((int64_t)row_end[mid] > p) hi = mid; else lo = mid + 1;
         }
         const int64_t src = p + shift[lo];
-        s_idx[p] = idx[src];
+        if (s_idx) s_idx[p] = idx[src];              // null: only the values are gathered
         s_val[p] = val[src];
     }
 }
@@ -543,7 +543,8 @@ __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
 // col_group(column, row_groups(degree)), stably inside each group, so that a
 // work unit of such a row touches rows of X that belong to one column group.
 // One workgroup per split row; counts[lr*64 + g] receives the size of each group
-// (counts may be null).
+// (counts may be null).  With s_idx null only the values are written (the columns of the
+// sorted copy are in place already and only the values changed).
 // ---------------------------------------------------------------------------
 constexpr int kGroupRound = 4;   // elements per thread between two barriers of group_long_rows_kernel
 
@@ -613,7 +614,7 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
 #pragma unroll
                 for (int q = 0; q < kThreads / 64; q++) pos += wave_cnt[flip][e2][q][g[e]];
             for (int q = 0; q < w; q++) pos += wave_cnt[flip][e][q][g[e]];
-            s_idx[dst0 + pos] = col[e];
+            if (s_idx) s_idx[dst0 + pos] = col[e];
             s_val[dst0 + pos] = v[e];
         }
         __syncthreads();
@@ -684,7 +685,7 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_wave_kernel(
         if (valid) pos = my[g] + rank;
         __builtin_amdgcn_wave_barrier();
         if (valid) {
-            s_idx[dst0 + pos] = col;
+            if (s_idx) s_idx[dst0 + pos] = col;
             s_val[dst0 + pos] = v;
             if (rank == 0) my[g] += __popcll(peers);     // one lane per group present
         }
@@ -1403,8 +1404,8 @@ int hash_words_device(const void *words_dev, int64_t n, uint64_t seed, uint64_t 
 // (s_idx, s_val), in place: rows that stay whole keep the order of their non-zeros, split rows
 // are regrouped by column group.  Needs perm (or identity_perm), s_indptr, nnz_short,
 // n_split_rows, n_wide_rows and plan_groups.  This is also how new values on an unchanged
-// structure reach the copy the kernels read.
-int refresh_sorted_csr(accel_handle *h, hipStream_t s)
+// structure reach the copy the kernels read (values_only: the columns are left as they are).
+int refresh_sorted_csr(accel_handle *h, bool values_only, hipStream_t s)
 {
     if (!h->owns_sorted) {                  // the sorted copy is the caller's CSR itself
         h->s_idx = h->idx;
@@ -1413,12 +1414,13 @@ int refresh_sorted_csr(accel_handle *h, hipStream_t s)
     }
     const int64_t rows = h->rows, n_long = h->n_split_rows, first_long = rows - n_long;
     const int64_t nnz_short = h->nnz_short;
-    int32_t *sidx = const_cast<int32_t *>(h->s_idx);
+    int32_t *sidx = values_only ? nullptr : const_cast<int32_t *>(h->s_idx);
     float *sval = const_cast<float *>(h->s_val);
     DevBuf tiles;
     if (nnz_short > 0) {
         if (h->identity_perm) {
-            ACCEL_HIP(hipMemcpyAsync(sidx, h->idx, sizeof(int32_t) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
+            if (sidx)
+                ACCEL_HIP(hipMemcpyAsync(sidx, h->idx, sizeof(int32_t) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
             ACCEL_HIP(hipMemcpyAsync(sval, h->val, sizeof(float) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
         } else {
             if (int rc = tiles.alloc(sizeof(int) * (size_t)(nnz_short / kPermuteTile + 2))) return rc;
@@ -1449,7 +1451,7 @@ int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s)
         h->s_idx = static_cast<int32_t *>(sidx.release());
         h->s_val = static_cast<float *>(sval.release());
     }
-    return refresh_sorted_csr(h, s);        // on failure release_products frees what was allocated
+    return refresh_sorted_csr(h, false, s); // on failure release_products frees what was allocated
 }
 
 int preprocess_device(accel_handle *h)
