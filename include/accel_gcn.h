@@ -160,7 +160,11 @@ int accel_load_state(accel_handle *h, const char *path);
  * the values into its own array; a handle that borrows device arrays needs a device
  * array and borrows that one from now on (it may be the same array, rewritten in
  * place).  Synchronous, and it waits for all work on the device first: do not call it
- * while a stream is capturing.  A saved state holds no values and stays valid. */
+ * while a stream is capturing.  A saved state holds no values and stays valid.  The
+ * sorted copy is rewritten where it is, so HIP graphs captured from runs of this handle
+ * stay valid and compute with the new values (exception: a CSR that was already sorted
+ * and has no split row is read in place, so passing a different array changes the
+ * address a captured run reads). */
 int accel_update_values(accel_handle *h, const float *val, int flags);
 
 /* Column panels (no counterpart upstream, which always walks all N columns of a row

@@ -117,6 +117,40 @@ def test_graph_capture_and_replay(gpu, hip):
     dX.close(); dY.close(); op.close()
 
 
+def test_captured_graph_sees_updated_values(gpu, hip):
+    """accel_update_values rewrites the sorted copy in place: a graph captured before the
+    update computes with the new values when it is replayed."""
+    g, X, op = make_case(gpu, 35, 48)
+    N = 48
+    assert op.info.n_split_rows > 0
+    dX, dY = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer(g.n_rows * N * 4)
+    op.run(dX, dY, N)
+    op.synchronize()
+    s = C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(s)))
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamBeginCapture(s, 0))
+    op.run(dX, dY, N, stream=s.value)
+    ok(hip.hipStreamEndCapture(s, C.byref(graph)))
+    ok(hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0))
+    for seed in (1, 2, 3):
+        v = np.random.default_rng(seed).uniform(-1, 1, g.values.size).astype(np.float32)
+        op.update_values(v)
+        dY.fill_u32(0x7FC00000)
+        op.synchronize()
+        ok(hip.hipGraphLaunch(gexec, s))
+        ok(hip.hipStreamSynchronize(s))
+        Y = dY.to_numpy(np.float32, (g.n_rows, N))
+        assert so.check(Y, g.indptr, g.indices, v, X) <= so.TOL, f"replay after update {seed}"
+        op.run(dX, dY, N)
+        op.synchronize()
+        assert np.array_equal(Y, dY.to_numpy(np.float32, (g.n_rows, N)))   # eager run: same bits
+    ok(hip.hipGraphExecDestroy(gexec))
+    ok(hip.hipGraphDestroy(graph))
+    ok(hip.hipStreamDestroy(s))
+    dX.close(); dY.close(); op.close()
+
+
 def test_second_stream_is_refused_while_the_first_run_is_in_flight(gpu, hip):
     """The partial-sum buffer of a handle is shared by its runs: a run on another stream
     while the previous one has not finished is an error, not silent corruption."""
