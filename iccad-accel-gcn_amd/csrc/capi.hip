@@ -122,7 +122,7 @@ using namespace accel;
 extern "C" {
 
 const char *accel_last_error(void) { return get_error(); }
-int accel_version(void) { return 100; }
+int accel_version(void) { return 200; }   // 0.2.0: saved state, value updates, strided and static runs
 
 // ---------------------------------------------------------------------------
 // host utilities
