@@ -414,6 +414,30 @@ def test_plan_split_threshold(gpu, unit, split, team):
     op.close()
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_plan_options_in_combination(gpu, seed):
+    """Unit size, split threshold, column groups and who works on a unit, drawn together:
+    the metadata never moves, the plan stays a cover of the non-zeros, the product holds."""
+    from oracle import spmm_oracle as so
+    rng = np.random.default_rng(1000 + seed)
+    unit = int(rng.choice([16, 24, 48, 77, 128, 250, 384]))
+    split = int(rng.choice([16, 40, 96, 192, 300, 384]))
+    groups = int(rng.choice([0, 8, 16, 32, 64]))
+    team = int(rng.choice([1, 2]))
+    deg = helpers.degree_mix(seed=seed, n_long=int(rng.integers(0, 8)), zeros=int(rng.integers(0, 9)))
+    if seed % 4 == 3:
+        deg = np.concatenate([deg, [int(rng.integers(5000, 30000))]])      # one hub row
+    g = helpers.graph_from_degrees(deg, seed=seed)
+    op = check_preprocess(gpu, g, plan_unit=unit, plan_split=split, plan_groups=groups or None, plan_team=team)
+    check_plan(op, g.n_cols)
+    for N in (int(rng.choice([1, 7, 20])), int(rng.choice([64, 100, 130]))):
+        X = np.random.default_rng(seed + N).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+        Y = op.matmul(X)
+        assert np.isfinite(Y).all()
+        assert so.check(Y, g.indptr, g.indices, g.values, X) <= so.TOL, (unit, split, groups, team, N)
+    op.close()
+
+
 def test_device_plumbing(gpu):
     import ctypes as C
     a = np.arange(100_003, dtype=np.uint32)
