@@ -42,6 +42,12 @@ class Info(C.Structure):
                 ("plan_split_nz", C.c_int32), ("plan_team", C.c_int32)]
 
 
+class RunArgs(C.Structure):
+    """accel_run_args of include/accel_gcn.h."""
+    _fields_ = [("X", C.c_void_p), ("Y", C.c_void_p), ("N", C.c_int32), ("ld", C.c_int32),
+                ("bias", C.c_void_p), ("flags", C.c_int32), ("stream", C.c_void_p)]
+
+
 i32p = C.POINTER(C.c_int32)
 f32p = C.POINTER(C.c_float)
 i64p = C.POINTER(C.c_int64)
@@ -82,6 +88,7 @@ SIGNATURES = {
     "accel_get_perm": (C.c_int, [vp, i32p, C.c_int64]),
     "accel_get_sorted_csr": (C.c_int, [vp, i32p, i32p, f32p]),
     "accel_run": (C.c_int, [vp, vp, vp, C.c_int32, vp]),
+    "accel_run_ex": (C.c_int, [vp, C.POINTER(RunArgs)]),
     "accel_run_strided": (C.c_int, [vp, vp, vp, C.c_int32, C.c_int32, vp]),
     "accel_reserve": (C.c_int, [vp, C.c_int32]),
     "accel_run_static": (C.c_int, [vp, vp, vp, C.c_int32, vp]),

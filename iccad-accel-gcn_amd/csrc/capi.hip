@@ -668,6 +668,18 @@ int accel_run_strided(accel_handle *h, const float *X, float *Y, int32_t N, int3
     return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, nullptr, 0, false, ld);
 }
 
+int accel_run_ex(accel_handle *h, const accel_run_args *a)
+{
+    clear_error();
+    if (!a) { set_error("accel_run_ex: null arguments"); return ACCEL_ERR_ARG; }
+    const int32_t ld = a->ld == 0 ? a->N : a->ld;
+    if (ld < a->N) { set_error("accel_run_ex: the row stride (%d) must be 0 or at least N (%d)", a->ld, a->N); return ACCEL_ERR_ARG; }
+    if (a->flags & ~ACCEL_EPILOGUE_RELU) { set_error("accel_run_ex: unknown flags %d", a->flags); return ACCEL_ERR_ARG; }
+    if (int rc = check_run(h, a->X, a->Y, a->N, a->bias, "accel_run_ex", ld)) return rc;
+    return spmm_launch(h, a->X, a->Y, a->N, static_cast<hipStream_t>(a->stream), nullptr, a->bias,
+                       (a->flags & ACCEL_EPILOGUE_RELU) ? 1 : 0, false, ld);
+}
+
 int accel_reserve(accel_handle *h, int32_t max_N)
 {
     clear_error();

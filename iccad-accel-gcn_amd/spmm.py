@@ -198,6 +198,22 @@ class AccelSpMM:
         check(lib().accel_run_epilogue(self._h, x, y, int(N), b,
                                        _lib.EPILOGUE_RELU if relu else 0, ptr(stream)))
 
+    def run_ex(self, X, Y, N: int, ld: int = 0, bias=None, relu=False, stream=None) -> None:
+        """Every option of a run at once (see accel_run_ex): rows ``ld`` floats apart
+        (0: packed), Y = act(A X + bias)."""
+        N, ld = int(N), int(ld)
+        step = ld or N
+        if N <= 0 or step < N:
+            raise AccelError(_lib.ERR_ARG, f"need 0 < N <= ld (or ld = 0), got N={N}, ld={ld}")
+        a = _lib.RunArgs()
+        x = _lib.dev_ptr(X, ((self.n_cols - 1) * step + N) * 4 if self.n_cols else 0, "X")
+        y = _lib.dev_ptr(Y, ((self.n_rows - 1) * step + N) * 4 if self.n_rows else 0, "Y")
+        b = _lib.dev_ptr(bias, N * 4, "bias")
+        s = ptr(stream)
+        a.X, a.Y, a.N, a.ld = x.value if x else None, y.value if y else None, N, ld
+        a.bias, a.flags, a.stream = b.value if b else None, _lib.EPILOGUE_RELU if relu else 0, s.value if s else None
+        check(lib().accel_run_ex(self._h, C.byref(a)))
+
     def synchronize(self, stream=None) -> None:
         check(lib().accel_stream_sync(ptr(stream)))
 

@@ -255,6 +255,23 @@ int accel_run_epilogue(accel_handle *h, const float *X, float *Y, int32_t N, con
  * written.  The partial-sum buffer is sized for ld (accel_reserve(h, ld)). */
 int accel_run_strided(accel_handle *h, const float *X, float *Y, int32_t N, int32_t ld, void *stream);
 
+/* The run with every option at once: rows `ld` floats apart (0 = packed, ld = N), bias
+ * and/or ReLU in the store, on `stream`.  accel_run, accel_run_epilogue and
+ * accel_run_strided are this call with the other fields left at zero; what it adds is
+ * their combination (a GCN layer on a padded feature matrix: Y = relu(A X + b) with rows
+ * a multiple of 32 floats apart).  No counterpart upstream, whose launch has one form
+ * (spmm_accel.cu:104-108). */
+typedef struct accel_run_args {
+    const float *X;    /* cols x N floats, rows ld apart */
+    float *Y;          /* rows x N floats, rows ld apart */
+    int32_t N;         /* columns computed */
+    int32_t ld;        /* floats between rows of X and of Y; 0 = N */
+    const float *bias; /* N floats on the device, or NULL */
+    int32_t flags;     /* 0 or ACCEL_EPILOGUE_RELU */
+    void *stream;      /* hipStream_t; NULL = default stream */
+} accel_run_args;
+int accel_run_ex(accel_handle *h, const accel_run_args *args);
+
 /* accel_run keeps the partial sums of split rows (pieces x N floats) in a buffer of the
  * handle.  It is allocated by the first accel_run with a given N and replaced by a larger
  * one when a later run brings a larger N; a HIP graph captured with the old buffer must

@@ -93,6 +93,60 @@ def test_rows_with_a_stride(gpu, mixed, N, ld):
     dY.close()
 
 
+@pytest.mark.parametrize("N,ld,relu", [(50, 64, True), (127, 128, False), (64, 0, True), (20, 32, True), (130, 160, True)])
+def test_every_option_of_a_run_at_once(gpu, mixed, N, ld, relu):
+    """accel_run_ex: rows with a stride and the fused bias / ReLU in one call; with the other
+    fields at zero it is accel_run / accel_run_strided / accel_run_epilogue, bit for bit."""
+    g, op = mixed
+    step = ld or N
+    rng = np.random.default_rng(N + step)
+    X = rng.uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    bias = rng.uniform(-0.5, 0.5, N).astype(np.float32)
+    Xp = np.full((g.n_cols, step), np.nan, np.float32)
+    Xp[:, :N] = X
+    dX = gpu.DeviceBuffer.from_numpy(Xp.reshape(-1)[: (g.n_cols - 1) * step + N])
+    dB = gpu.DeviceBuffer.from_numpy(bias)
+    n_out = (g.n_rows - 1) * step + N
+
+    def result(call):
+        dY = gpu.DeviceBuffer(n_out * 4)
+        dY.fill_u32(0x7FC00000)
+        call(dY)
+        op.synchronize()
+        Yp = np.full((g.n_rows, step), np.nan, np.float32)
+        Yp.reshape(-1)[:n_out] = dY.to_numpy(np.float32, (n_out,))
+        dY.close()
+        assert np.isnan(Yp[:-1, N:]).all(), "padding columns of Y were written"
+        return np.ascontiguousarray(Yp[:, :N])
+
+    Y = result(lambda dY: op.run_ex(dX, dY, N, ld=ld, bias=dB, relu=relu))
+    R, S = so.spmm_fp64(g.indptr, g.indices, g.values, X)
+    R = R + bias.astype(np.float64)
+    if relu:
+        R = np.maximum(R, 0.0)
+    assert np.isfinite(Y).all()
+    assert np.max(np.abs(Y - R) / np.maximum(S + np.abs(bias), 1e-30)) <= TOL
+    if relu:
+        assert (Y >= 0).all()
+    # the plain product through the same entry point = the dedicated entry points
+    plain = result(lambda dY: op.run_ex(dX, dY, N, ld=ld))
+    same = result(lambda dY: op.run_strided(dX, dY, N, step)) if ld else result(lambda dY: op.run(dX, dY, N))
+    assert np.array_equal(plain.view(np.uint32), same.view(np.uint32))
+    if not ld:
+        fused = result(lambda dY: op.run_epilogue(dX, dY, N, bias=dB, relu=relu))
+        assert np.array_equal(Y.view(np.uint32), fused.view(np.uint32))
+    with pytest.raises(gpu.AccelError) as e:
+        op.run_ex(dX, gpu.DeviceBuffer(16), N, ld=ld)          # Y too small
+    assert e.value.status == gpu._lib.ERR_ARG
+    L = gpu._lib.lib()
+    assert L.accel_run_ex(op._h, None) == gpu._lib.ERR_ARG
+    a = gpu._lib.RunArgs()
+    a.X, a.N, a.ld, a.flags = dX.address, N, step, 8
+    assert L.accel_run_ex(op._h, a) == gpu._lib.ERR_ARG        # unknown flag (checked before Y)
+    dX.close()
+    dB.close()
+
+
 @pytest.mark.parametrize("N", [17, 33, 50, 99, 127])
 def test_column_counts_of_upstreams_sweep_on_cfg2(gpu, N):
     """Upstream sweeps dim 16..128 in steps of 1 (main.cu:12): three quarters of those are
