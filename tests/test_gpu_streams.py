@@ -18,7 +18,7 @@ def hip(gpu):
     h = C.CDLL("libamdhip64.so.7")
     for name in ("hipStreamCreate", "hipStreamDestroy", "hipStreamSynchronize", "hipStreamBeginCapture",
                  "hipStreamEndCapture", "hipGraphInstantiate", "hipGraphLaunch", "hipGraphExecDestroy",
-                 "hipGraphDestroy"):
+                 "hipGraphDestroy", "hipMemGetInfo", "hipDeviceSynchronize"):
         getattr(h, name).restype = C.c_int
     return h
 
@@ -289,3 +289,45 @@ def test_no_device_memory_leak(gpu, hip):
     gpu._lib.check(gpu.lib().accel_stream_sync(None))
     ok(hip.hipMemGetInfo(C.byref(free1), C.byref(total)))
     assert free0.value - free1.value < (8 << 20), f"free memory fell by {free0.value - free1.value} bytes"
+
+
+def test_handles_give_their_memory_back(gpu, hip, tmp_path):
+    """Create, preprocess (or load a state), run every way, update the values, destroy,
+    many times over: the free device memory must come back to where it was."""
+    g = gpu.synthetic.cfg2()                               # 2.4 M non-zeros: some 50 MB per handle
+    N = 64
+    X = gpu.synthetic.dense_operand("cfg2", g.n_cols, N)
+    dX, dY = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer(g.n_rows * N * 4)
+    state = tmp_path / "cfg2.accelstate"
+
+    def free_bytes():
+        ok(hip.hipDeviceSynchronize())
+        free, total = C.c_size_t(), C.c_size_t()
+        ok(hip.hipMemGetInfo(C.byref(free), C.byref(total)))
+        return free.value
+
+    def cycle(i):
+        op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols)
+        if i % 3 == 2:
+            op.load_state(state)
+        else:
+            op.preprocess()
+        if i == 0:
+            op.save_state(state)
+        op.run(dX, dY, N)
+        op.reserve(128)
+        op.run_static(dX, dY, 16)
+        op.run_ex(dX, dY, 32, ld=64, relu=True)
+        op.update_values(g.values)
+        if i % 4 == 1:
+            op.preprocess()                                # a second time on the same handle
+        op.synchronize()
+        op.close()
+
+    cycle(0)                                               # whatever the first use of the library keeps
+    before = free_bytes()
+    for i in range(1, 25):
+        cycle(i)
+    after = free_bytes()
+    assert before - after < 8 << 20, f"{(before - after) / 1e6:.1f} MB not returned after 24 handles"
+    dX.close(); dY.close()
