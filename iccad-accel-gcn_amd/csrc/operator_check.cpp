@@ -81,6 +81,30 @@ int main()
     bad.set_meta_dir("/nonexistent/");
     if (bad.do_test(false, 4) >= 0) return fail("host pointer as vout was accepted");
     std::printf("ok: host pointer refused (%s)\n", bad.error().c_str());
+    // values rewritten between two calls: the second call computes with the new ones, also when
+    // the operator works from a degree-sorted copy (rows here are in descending degree order)
+    {
+        const std::vector<int> rptr_h = {0, 3, 6, 8, 9, 10, 10};
+        const std::vector<int> ridx_h = {1, 3, 5, 0, 2, 4, 1, 5, 0, 3};
+        for (int i = 0; i <= v_num; i++) ptr[i] = rptr_h[i];
+        for (int i = 0; i < e_num; i++) { idx[i] = ridx_h[i]; val[i] = 1.0f + (float)i; }
+        SPMM_ACCEL again("check", ptr, idx, val, vin, vout, v_num, e_num, dim_max);
+        again.set_meta_dir("/nonexistent/");
+        for (int pass = 0; pass < 2; pass++) {
+            if (pass == 1)
+                for (int i = 0; i < e_num; i++) val[i] = 0.5f * (float)(e_num - i);
+            if (again.do_test(false, 4) != 0.0) return fail("do_test on the unsorted matrix");
+            for (int r = 0; r < v_num; r++)
+                for (int c = 0; c < 4; c++) {
+                    float want = 0.0f;
+                    for (int p = ptr[r]; p < ptr[r + 1]; p++) want += val[p] * vin[idx[p] * 4 + c];
+                    if (std::fabs(vout[r * 4 + c] - want) > 1e-4f * (1.0f + std::fabs(want)))
+                        return fail(pass ? "values rewritten between two calls were not picked up"
+                                         : "wrong product on the unsorted matrix");
+                }
+        }
+        std::printf("ok: values rewritten between two do_test calls are used\n");
+    }
     (void)hipFree(ptr); (void)hipFree(idx); (void)hipFree(val); (void)hipFree(vin); (void)hipFree(vout);
     return 0;
 }

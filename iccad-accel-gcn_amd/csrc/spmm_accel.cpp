@@ -12,7 +12,16 @@ SPMM_ACCEL::~SPMM_ACCEL()
 
 bool SPMM_ACCEL::preprocess()
 {
-    if (h) return true;
+    if (h) {
+        // Upstream's kernel reads val on every launch (spmm_accel.cu:75), so a caller that
+        // rewrote the array between two do_test calls computes with the new values; the
+        // sorted copy this operator computes from is brought up to date the same way.
+        if (accel_update_values(h, val, ACCEL_PTR_DEVICE) != ACCEL_OK) {
+            err = accel_last_error();
+            return false;
+        }
+        return true;
+    }
     err.clear();
     int rc = accel_create(ptr, idx, val, num_v, num_v, num_e, ACCEL_PTR_DEVICE, &h);
     if (!rc) {

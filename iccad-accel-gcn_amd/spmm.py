@@ -269,7 +269,7 @@ class SpmmAccel:
 
     def __init__(self, graph, ptr_, idx, val, vin, vout, num_v, num_e, dim, meta_dir="../block_level_meta/"):
         self._graph = graph
-        self.vin, self.vout = vin, vout
+        self.val, self.vin, self.vout = val, vin, vout
         self.num_v, self.num_e, self.dim = int(num_v), int(num_e), int(dim)
         self.meta_dir = Path(meta_dir)
         self.save_state = False        # True: write <meta_dir>/<graph>.accelstate after preprocessing
@@ -279,6 +279,9 @@ class SpmmAccel:
 
     def _preprocess(self):
         if self._ready:
+            # upstream's kernel reads val on every launch (spmm_accel.cu:75): a caller may have
+            # rewritten the array since the last call
+            self._op.update_values(self.val)
             return
         # the saved state of an earlier run takes the place of the preprocessing, as
         # upstream's operator loads its metadata file (spmm_accel.cu:122); a state that

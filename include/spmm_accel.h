@@ -12,6 +12,8 @@
  * sort and the metadata are built on the GPU once and cached in the object.  If
  * that file exists it is compared with the GPU-built metadata and a mismatch is
  * an error (do_test returns -1), so a stale file cannot silently mis-index.
+ * The values are read again on every do_test (upstream's kernel reads val on every
+ * launch, spmm_accel.cu:75): a caller may rewrite val between two calls.
  * run(dim): one asynchronous launch; vout = A * vin with leading dimension dim.
  * After a launch has failed, run() launches nothing more and do_test returns -1.
  *

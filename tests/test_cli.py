@@ -43,12 +43,13 @@ def test_cli_without_gpu_says_so(pkg):
 @pytest.mark.gpu
 def test_operator_error_paths(gpu):
     """bin/operator_check: a refused launch is reported by do_test and nothing more is
-    launched, the operator computes again afterwards, a host pointer is refused."""
+    launched, the operator computes again afterwards, a host pointer is refused, values
+    rewritten between two calls are picked up."""
     exe = EXE.parent / "operator_check"
     assert exe.exists(), "operator_check was not built"
     r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("ok:") == 4 and "FAIL" not in r.stdout
+    assert r.stdout.count("ok:") == 5 and "FAIL" not in r.stdout
 
 
 @pytest.mark.gpu

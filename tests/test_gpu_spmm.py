@@ -312,6 +312,13 @@ def test_operator_mirror_do_test(gpu, tmp_path):
         assert so.check(Y, sip, six, sval, Xd) <= TOL
     t = acc.do_test(True, 64)
     assert 0 < t < 1.0
+    # the array of values rewritten in place between two calls (upstream's kernel reads it on
+    # every launch, spmm_accel.cu:75): the next call computes with the new values
+    v2 = (sval * np.float32(-0.5)).astype(np.float32)
+    gpu._lib.check(gpu._lib.lib().accel_memcpy_h2d(bufs[2].address, v2.ctypes.data, v2.nbytes))
+    assert acc.do_test(False, 16) == 0.0
+    Xd = X.reshape(-1)[: g0.n_cols * 16].reshape(g0.n_cols, 16)
+    assert so.check(vout.to_numpy(np.float32, (g0.n_rows, 16)), sip, six, v2, Xd) <= TOL
     b = po.partition_closed_form(sip).copy()
     b[0, 3] += 1
     gpu.block_level_partition.write_block4(meta / "stale.block4", b)
