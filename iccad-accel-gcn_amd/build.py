@@ -82,13 +82,6 @@ def build_baselines(verbose: bool = False) -> Path:
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for baselines/*.cpp:\n" + r.stdout)
-    # a stand-alone probe (see its header): bin/band_sweep_probe
-    BIN_DIR.mkdir(exist_ok=True)
-    cmd = [hipcc(), *compile_flags(), str(PKG / "baselines" / "band_sweep_probe.cpp"), "-o",
-           str(BIN_DIR / "band_sweep_probe")]
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("hipcc failed for baselines/band_sweep_probe.cpp:\n" + r.stdout)
     return out
 
 

@@ -9,12 +9,21 @@
  * timed on the host with a device synchronisation, arithmetic mean in seconds,
  * 0 when timing is off (:34-63).  The only change is the runtime: HIP's dim3 and
  * hipDeviceSynchronize, and a steady clock instead of system_clock (util.h:4-9).
+ *
+ * What a translation unit gets from including this file is part of the
+ * interface too: upstream's header pulls in util.h (:2, the timestamp /
+ * getDuration helpers) and <string> and opens namespace std (:4), and its own
+ * caller relies on that (main.cu:10 names `string` before its own using-
+ * directive).  This header does the same.
  */
 #pragma once
 #include <hip/hip_runtime.h>
 
 #include <chrono>
 #include <string>
+
+#include "util.h"
+using namespace std;
 
 class SPMM_BASE
 {

@@ -1,10 +1,11 @@
-"""Writes upstream_degrees.json: the degree sequence of each of the reference's
-benchmark graphs, as (degree, row count) pairs in ascending degree order.
+"""Writes iccad-accel-gcn_amd/data/upstream_degrees.json: the degree sequence of each
+of the reference's benchmark graphs, as (degree, row count) pairs in ascending degree
+order.
 
-The sequences are read out of the golden ``.block4`` metadata kept under
-tests/golden (degree, first row and row count of every block; rows that no block
-covers have degree 0).  Run from the repository root:
-    python iccad-accel-gcn_amd/data/make_upstream_degrees.py
+The sequences are read out of the golden ``.block4`` metadata kept next to this
+script (degree, first row and row count of every block; rows that no block covers
+have degree 0).  Run from the repository root:
+    python tests/golden/make_upstream_degrees.py
 """
 import json
 import sys
@@ -13,7 +14,7 @@ from pathlib import Path
 import numpy as np
 
 ROOT = Path(__file__).resolve().parents[2]
-sys.path.insert(0, str(ROOT / "tests" / "golden"))
+sys.path.insert(0, str(Path(__file__).resolve().parent))
 import block4_codec  # noqa: E402
 
 
@@ -37,7 +38,7 @@ def main():
     for name in block4_codec.names():
         d, c = np.unique(degrees(block4_codec.load(name)), return_counts=True)
         out[name] = [[int(a), int(b)] for a, b in zip(d, c)]
-    path = Path(__file__).resolve().parent / "upstream_degrees.json"
+    path = ROOT / "iccad-accel-gcn_amd" / "data" / "upstream_degrees.json"
     path.write_text(json.dumps(out, separators=(",", ":")) + "\n")
     print(path, path.stat().st_size, "bytes")
 

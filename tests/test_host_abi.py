@@ -175,3 +175,21 @@ def test_binding_refuses_host_arrays_as_dense_operands(pkg):
     assert L.dev_ptr(FakeTensor(8, True), 32, "Y").value == 0x1000
     assert L.dev_ptr(None, 4, "bias") is None
     assert L.dev_ptr(0x2000, 1 << 40, "X").value == 0x2000  # raw addresses are the library's to check
+
+
+def test_upstream_shaped_caller_compiles_against_the_headers(pkg, tmp_path):
+    """A driver with the shape of upstream's main.cu (`string` named before its own
+    using-directive, main.cu:10,16; the readers of data.h; the nine-argument constructor,
+    main.cu:131; do_test(false/true, dim), main.cu:146,166; the host-clock helpers of
+    util.h) builds against include/ alone and links against the library."""
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    src = ROOT / "tests" / "cases" / "upstream_shaped_caller.cpp"
+    lib_dir = Path(pkg._lib.LIB_PATH).parent
+    exe = tmp_path / "caller"
+    r = subprocess.run([hipcc, "-x", "hip", "--offload-arch=gfx950", "-std=c++17", "-Wno-unused-value",
+                        f"-I{ROOT / 'include'}", str(src), "-o", str(exe), f"-L{lib_dir}", "-laccelgcn"],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert exe.exists()
