@@ -25,6 +25,7 @@ void clear_error() { g_error.clear(); }
 
 int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
                           int32_t **block4_dev, int64_t *n_blocks);
+bool stream_is_capturing(hipStream_t s);
 
 void release_products(accel_handle *h)
 {
@@ -43,8 +44,17 @@ void release_products(accel_handle *h)
     if (h->long_slot) (void)hipFree(h->long_slot);
     if (h->block4) (void)hipFree(h->block4);
     if (h->partial) (void)hipFree(h->partial);
-    if (h->partial_done) (void)hipEventDestroy(h->partial_done);
-    h->partial_done = nullptr; h->partial_stream = nullptr; h->partial_in_use = false;
+    if (h->src_pos) (void)hipFree(h->src_pos);
+    h->src_pos = nullptr;
+    // what other streams still hold was queued against the memory freed above (hipFree waits
+    // for the device), so the bookkeeping starts afresh
+    if (h->writer_done) (void)hipEventDestroy(h->writer_done);
+    for (auto &sl : h->slot) {
+        if (sl.done) (void)hipEventDestroy(sl.done);
+        sl = accel_handle::StreamSlot();
+    }
+    h->writer_done = nullptr; h->writer = nullptr; h->writer_pending = false;
+    h->partial_slot = -1; h->next_victim = 0; h->track_runs = false;
     h->perm = nullptr; h->s_indptr = nullptr; h->s_idx = nullptr; h->s_val = nullptr;
     h->work = nullptr; h->long_slot = nullptr; h->block4 = nullptr; h->partial = nullptr;
     h->n_units = h->n_long_units = 0;
@@ -66,15 +76,21 @@ static int need_gpu()
 
 // A dense operand must be memory the GPU can read: a host address handed to a kernel is a
 // memory fault, not an error code.  The runtime is asked what the address is and, where it
-// knows the allocation, whether `bytes` fit behind it.  Each (address, size) that passed is
-// remembered, so the check costs nothing in a loop over the same buffers.
-static int check_operand(accel_handle *h, const void *p, size_t bytes, const char *fn, const char *name)
+// knows the allocation, whether `bytes` fit behind it.  It is asked on every call: an answer
+// remembered from an earlier call says nothing once the caller has freed the buffer and a
+// smaller one has taken its address (allocators that recycle addresses do this all the time).
+// Not while a stream is capturing: the runtime counts these queries among the calls that
+// end a capture in error, so a captured run takes its operands unchecked (check_run).
+static int check_operand(const void *p, size_t bytes, const char *fn, const char *name)
 {
     if (!p || bytes == 0) return ACCEL_OK;
-    for (const auto &c : h->checked)
-        if (c.p == p && c.bytes >= bytes) return ACCEL_OK;
     hipPointerAttribute_t at;
-    if (hipPointerGetAttributes(&at, p) != hipSuccess || at.type == hipMemoryTypeUnregistered) {
+    const hipError_t qe = hipPointerGetAttributes(&at, p);
+    if (qe == hipErrorStreamCaptureUnsupported || qe == hipErrorStreamCaptureImplicit) {
+        (void)hipGetLastError();            // another stream of this process is capturing: nothing can be asked
+        return ACCEL_OK;
+    }
+    if (qe != hipSuccess || at.type == hipMemoryTypeUnregistered) {
         (void)hipGetLastError();
         set_error("%s: %s (%p) is not memory the GPU can access (a host array? copy it to the device first)",
                   fn, name, p);
@@ -92,27 +108,134 @@ static int check_operand(accel_handle *h, const void *p, size_t bytes, const cha
     } else {
         (void)hipGetLastError();
     }
-    h->checked[h->checked_next] = {p, bytes};
-    h->checked_next = (h->checked_next + 1) % 4;
+    return ACCEL_OK;
+}
+
+// The handle's device memory belongs to the GPU it was created on; a launch with another GPU
+// current would hand that GPU addresses it cannot use.
+static int check_device(const accel_handle *h, const char *fn)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); dev = -1; }
+    if (dev != h->device) {
+        set_error("%s: the handle was created on GPU %d, the current device is %d (hipSetDevice(%d) first)", fn,
+                  h->device, dev, h->device);
+        return ACCEL_ERR_STATE;
+    }
     return ACCEL_OK;
 }
 
 // argument checks shared by the run entry points
 static int check_run(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias, const char *fn,
-                     int32_t ld = 0)
+                     hipStream_t stream, int32_t ld = 0)
 {
     if (!h) { set_error("%s: null handle", fn); return ACCEL_ERR_ARG; }
     if (!h->ready) { set_error("%s: call accel_preprocess first", fn); return ACCEL_ERR_STATE; }
     if (N <= 0) { set_error("%s: N must be positive, got %d", fn, N); return ACCEL_ERR_ARG; }
+    if (int rc = check_device(h, fn)) return rc;
     if ((h->rows > 0 && !Y) || (h->nnz > 0 && !X)) { set_error("%s: null dense operand", fn); return ACCEL_ERR_ARG; }
     if (h->rows == 0) return ACCEL_OK;
+    if (stream_is_capturing(stream)) return ACCEL_OK;    // see check_operand
     if (ld <= 0) ld = N;
     // the last row only has to hold N floats
     const size_t x_floats = h->cols > 0 ? (size_t)(h->cols - 1) * (size_t)ld + (size_t)N : 0;
     const size_t y_floats = (size_t)(h->rows - 1) * (size_t)ld + (size_t)N;
-    if (int rc = check_operand(h, X, x_floats * sizeof(float), fn, "X")) return rc;
-    if (int rc = check_operand(h, Y, y_floats * sizeof(float), fn, "Y")) return rc;
-    return check_operand(h, bias, (size_t)N * sizeof(float), fn, "bias");
+    if (int rc = check_operand(X, x_floats * sizeof(float), fn, "X")) return rc;
+    if (int rc = check_operand(Y, y_floats * sizeof(float), fn, "Y")) return rc;
+    return check_operand(bias, (size_t)N * sizeof(float), fn, "bias");
+}
+
+// ---------------------------------------------------------------------------
+// Stream order of a handle's mutable device memory.  Runs read the sorted values and, when
+// the matrix has split rows, write and then read the partial-sum buffer; a value update
+// rewrites the sorted values.  Work queued on one stream is ordered by the stream.  Across
+// streams the handle orders it itself, on the device, without making the host wait: a
+// tracked run binds an event to its last kernel (no extra packet in the queue), kept in the
+// slot of its stream, and whatever has to come after that run on another stream waits for
+// the event.  Runs are tracked when the matrix has split rows (the shared buffer) and, from
+// the first value update on, always.  A stream is never touched after the call that used it
+// has returned, so the caller may destroy it at any time.  A stream that is capturing is
+// left alone (an event of work outside a capture cannot be waited for inside one): the
+// caller orders a graph against other uses of the handle.
+// ---------------------------------------------------------------------------
+bool stream_is_capturing(hipStream_t s)
+{
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return cap != hipStreamCaptureStatusNone;
+}
+
+// Before a run is queued on s.  *run_done receives the event to bind to the run's last kernel
+// (null: this run is not tracked).
+int order_run(accel_handle *h, hipStream_t s, bool uses_partial, bool capturing, hipEvent_t *run_done)
+{
+    *run_done = nullptr;
+    if (capturing) return ACCEL_OK;
+    if (h->writer_pending && s != h->writer) {
+        if (hipEventQuery(h->writer_done) == hipSuccess) {
+            h->writer_pending = false;
+        } else {
+            (void)hipGetLastError();
+            ACCEL_HIP(hipStreamWaitEvent(s, h->writer_done, 0));
+        }
+    }
+    if (!uses_partial && !h->track_runs) return ACCEL_OK;
+    int mine = -1;
+    for (int i = 0; i < accel_handle::kMaxStreams; i++)
+        if (h->slot[i].done && h->slot[i].stream == s) mine = i;
+    if (mine < 0) {
+        for (int i = 0; i < accel_handle::kMaxStreams && mine < 0; i++)
+            if (!h->slot[i].done) mine = i;
+        if (mine < 0) {
+            // a fifth stream: it takes over a slot and waits for what that slot's stream held,
+            // so that whoever waits for this run also waits for those
+            mine = h->next_victim;
+            h->next_victim = (h->next_victim + 1) % accel_handle::kMaxStreams;
+            ACCEL_HIP(hipStreamWaitEvent(s, h->slot[mine].done, 0));
+        } else {
+            ACCEL_HIP(hipEventCreateWithFlags(&h->slot[mine].done, hipEventDisableTiming));
+        }
+        h->slot[mine].stream = s;
+    }
+    if (uses_partial) {
+        if (h->partial_slot >= 0 && h->partial_slot != mine)
+            ACCEL_HIP(hipStreamWaitEvent(s, h->slot[h->partial_slot].done, 0));
+        h->partial_slot = mine;
+    }
+    h->slot[mine].live = true;
+    *run_done = h->slot[mine].done;
+    return ACCEL_OK;
+}
+
+// Before a value update is queued on s: it has to come after every run that reads the
+// values it rewrites, and after an earlier update on another stream.
+int order_update(accel_handle *h, hipStream_t s, bool capturing)
+{
+    if (capturing) return ACCEL_OK;
+    if (!h->track_runs) {
+        // the first update of this handle: its runs so far left no events behind
+        ACCEL_HIP(hipDeviceSynchronize());
+        h->track_runs = true;
+    }
+    for (auto &sl : h->slot)
+        if (sl.live && sl.stream != s) ACCEL_HIP(hipStreamWaitEvent(s, sl.done, 0));
+    if (h->writer_pending && h->writer != s) ACCEL_HIP(hipStreamWaitEvent(s, h->writer_done, 0));
+    return ACCEL_OK;
+}
+
+// Behind a value update queued on s.
+int note_update(accel_handle *h, hipStream_t s, bool capturing)
+{
+    if (capturing) return ACCEL_OK;
+    if (!h->writer_done) ACCEL_HIP(hipEventCreateWithFlags(&h->writer_done, hipEventDisableTiming));
+    ACCEL_HIP(hipEventRecord(h->writer_done, s));
+    h->writer = s;
+    h->writer_pending = true;
+    for (auto &sl : h->slot) sl.live = false;   // later runs order themselves behind this update
+    return ACCEL_OK;
 }
 
 }  // namespace accel
@@ -356,6 +479,10 @@ int accel_create(const int32_t *indptr, const int32_t *idx, const float *val, in
     if (!h) { set_error("host allocation failed"); return ACCEL_ERR_ALLOC; }
     h->rows = rows; h->cols = cols; h->nnz = nnz;
     (void)hipGetDevice(&h->device);
+    if (hipDeviceGetAttribute(&h->device_cus, hipDeviceAttributeMultiprocessorCount, h->device) != hipSuccess) {
+        (void)hipGetLastError();
+        h->device_cus = 0;
+    }
     if (flags == ACCEL_PTR_DEVICE) {
         h->indptr = indptr; h->idx = idx; h->val = val;
         h->owns_input = false;
@@ -452,6 +579,18 @@ int accel_set_plan_team(accel_handle *h, int mode)
     return ACCEL_OK;
 }
 
+int accel_set_plan_queues(accel_handle *h, int queues)
+{
+    clear_error();
+    if (!h) { set_error("accel_set_plan_queues: null handle"); return ACCEL_ERR_ARG; }
+    if (queues != 0 && queues != 1 && queues != kXcds) {
+        set_error("accel_set_plan_queues: queues must be 0 (from the device), 1 or %d, got %d", kXcds, queues);
+        return ACCEL_ERR_ARG;
+    }
+    h->plan_queues_option = queues;
+    return ACCEL_OK;
+}
+
 int accel_set_plan_panel(accel_handle *h, int columns)
 {
     clear_error();
@@ -475,6 +614,50 @@ int accel_preprocess(accel_handle *h)
     return rc;
 }
 
+// Common part of the two value updates: val_dev holds the new values on the device, in the
+// order of the caller's CSR; everything is queued on `stream`.
+static int update_values_on_stream(accel_handle *h, const float *val_dev, hipStream_t stream, const char *fn)
+{
+    (void)hipGetLastError();                // launch errors are read back below: start from a clean slate
+    const bool capturing = stream_is_capturing(stream);
+    if (h->owns_sorted && !h->src_pos) {
+        if (capturing) {
+            set_error("%s: the first value update of a handle builds its position map (one allocation); "
+                      "do it once before the capture", fn);
+            return ACCEL_ERR_STATE;
+        }
+        if (int rc = build_source_positions(h, stream)) return rc;
+    }
+    if (int rc = order_update(h, stream, capturing)) return rc;
+    if (h->owns_input) {
+        // the handle's own copy of the caller's values follows (a later accel_preprocess reads it)
+        if (val_dev != h->val)
+            if (int rc = copy_u32(const_cast<float *>(h->val), val_dev, (size_t)h->nnz, stream)) return rc;
+    } else {
+        h->val = val_dev;                   // borrowed from now on (it may be the same array, rewritten)
+    }
+    if (h->owns_sorted) {
+        if (int rc = gather_values(h, h->val, stream)) return rc;
+    } else {
+        h->s_val = h->val;                  // the kernels read the caller's order in place
+    }
+    return note_update(h, stream, capturing);
+}
+
+int accel_update_values_async(accel_handle *h, const float *val_dev, void *stream)
+{
+    clear_error();
+    if (!h) { set_error("accel_update_values_async: null handle"); return ACCEL_ERR_ARG; }
+    if (!h->ready) { set_error("accel_update_values_async: call accel_preprocess first"); return ACCEL_ERR_STATE; }
+    if (int rc = check_device(h, "accel_update_values_async")) return rc;
+    if (h->nnz == 0) return ACCEL_OK;
+    if (!val_dev) { set_error("accel_update_values_async: null array"); return ACCEL_ERR_ARG; }
+    if (!stream_is_capturing(static_cast<hipStream_t>(stream)))
+        if (int rc = check_operand(val_dev, sizeof(float) * (size_t)h->nnz, "accel_update_values_async", "val"))
+            return rc;
+    return update_values_on_stream(h, val_dev, static_cast<hipStream_t>(stream), "accel_update_values_async");
+}
+
 int accel_update_values(accel_handle *h, const float *val, int flags)
 {
     clear_error();
@@ -484,26 +667,32 @@ int accel_update_values(accel_handle *h, const float *val, int flags)
         set_error("accel_update_values: unknown flags %d", flags);
         return ACCEL_ERR_ARG;
     }
+    if (int rc = check_device(h, "accel_update_values")) return rc;
     if (h->nnz == 0) return ACCEL_OK;
     if (!val) { set_error("accel_update_values: null array"); return ACCEL_ERR_ARG; }
     const size_t bytes = sizeof(float) * (size_t)h->nnz;
     if (flags == ACCEL_PTR_DEVICE)
-        if (int rc = check_operand(h, val, bytes, "accel_update_values", "val")) return rc;
+        if (int rc = check_operand(val, bytes, "accel_update_values", "val")) return rc;
     if (!h->owns_input && flags != ACCEL_PTR_DEVICE) {
         set_error("accel_update_values: this handle borrows its CSR from device memory; pass the new "
                   "values as a device array (ACCEL_PTR_DEVICE)");
         return ACCEL_ERR_ARG;
     }
-    // runs of this handle that are still in flight read the arrays rewritten below
-    ACCEL_HIP(hipDeviceSynchronize());
-    if (h->owns_input) {
-        if (val != h->val)
-            ACCEL_HIP(hipMemcpy(const_cast<float *>(h->val), val, bytes,
-                                flags == ACCEL_PTR_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice));
-    } else {
-        h->val = val;                       // borrowed from now on (it may be the same array, rewritten)
+    hipStream_t s = nullptr;
+    if (stream_is_capturing(s)) {
+        set_error("accel_update_values waits for its own work; use accel_update_values_async in a capture");
+        return ACCEL_ERR_STATE;
     }
-    return refresh_sorted_csr(h, true, nullptr);
+    if (flags == ACCEL_PTR_HOST) {
+        // into the handle's own copy of the caller's order, behind the runs that may still read it
+        if (int rc = order_update(h, s, false)) return rc;
+        ACCEL_HIP(hipMemcpyAsync(const_cast<float *>(h->val), val, bytes, hipMemcpyHostToDevice, s));
+        val = h->val;
+    }
+    if (int rc = update_values_on_stream(h, val, s, "accel_update_values")) return rc;
+    ACCEL_HIP(hipStreamSynchronize(s));
+    h->writer_pending = false;
+    return ACCEL_OK;
 }
 
 int accel_get_info(const accel_handle *h, accel_info *out)
@@ -522,6 +711,7 @@ int accel_get_info(const accel_handle *h, accel_info *out)
     out->plan_groups = h->plan_groups;
     out->plan_split_nz = h->plan_split;
     out->plan_team = h->plan_team ? 1 : 0;
+    out->plan_queues = h->plan_queues;
     return ACCEL_OK;
 }
 
@@ -656,16 +846,16 @@ int accel_partition_gpu(const int32_t *indptr, int64_t rows, int32_t *block4_out
 int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream)
 {
     clear_error();
-    if (int rc = check_run(h, X, Y, N, nullptr, "accel_run")) return rc;
-    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr);
+    if (int rc = check_run(h, X, Y, N, nullptr, "accel_run", static_cast<hipStream_t>(stream))) return rc;
+    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream));
 }
 
 int accel_run_strided(accel_handle *h, const float *X, float *Y, int32_t N, int32_t ld, void *stream)
 {
     clear_error();
     if (ld < N) { set_error("accel_run_strided: the row stride (%d) must be at least N (%d)", ld, N); return ACCEL_ERR_ARG; }
-    if (int rc = check_run(h, X, Y, N, nullptr, "accel_run_strided", ld)) return rc;
-    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, nullptr, 0, false, ld);
+    if (int rc = check_run(h, X, Y, N, nullptr, "accel_run_strided", static_cast<hipStream_t>(stream), ld)) return rc;
+    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, 0, false, ld);
 }
 
 int accel_run_ex(accel_handle *h, const accel_run_args *a)
@@ -675,8 +865,8 @@ int accel_run_ex(accel_handle *h, const accel_run_args *a)
     const int32_t ld = a->ld == 0 ? a->N : a->ld;
     if (ld < a->N) { set_error("accel_run_ex: the row stride (%d) must be 0 or at least N (%d)", a->ld, a->N); return ACCEL_ERR_ARG; }
     if (a->flags & ~ACCEL_EPILOGUE_RELU) { set_error("accel_run_ex: unknown flags %d", a->flags); return ACCEL_ERR_ARG; }
-    if (int rc = check_run(h, a->X, a->Y, a->N, a->bias, "accel_run_ex", ld)) return rc;
-    return spmm_launch(h, a->X, a->Y, a->N, static_cast<hipStream_t>(a->stream), nullptr, a->bias,
+    if (int rc = check_run(h, a->X, a->Y, a->N, a->bias, "accel_run_ex", static_cast<hipStream_t>(a->stream), ld)) return rc;
+    return spmm_launch(h, a->X, a->Y, a->N, static_cast<hipStream_t>(a->stream), nullptr, nullptr, a->bias,
                        (a->flags & ACCEL_EPILOGUE_RELU) ? 1 : 0, false, ld);
 }
 
@@ -692,17 +882,17 @@ int accel_reserve(accel_handle *h, int32_t max_N)
 int accel_run_static(accel_handle *h, const float *X, float *Y, int32_t N, void *stream)
 {
     clear_error();
-    if (int rc = check_run(h, X, Y, N, nullptr, "accel_run_static")) return rc;
-    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, nullptr, 0, true);
+    if (int rc = check_run(h, X, Y, N, nullptr, "accel_run_static", static_cast<hipStream_t>(stream))) return rc;
+    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, 0, true);
 }
 
 int accel_run_epilogue(accel_handle *h, const float *X, float *Y, int32_t N, const float *bias,
                        int flags, void *stream)
 {
     clear_error();
-    if (int rc = check_run(h, X, Y, N, bias, "accel_run_epilogue")) return rc;
+    if (int rc = check_run(h, X, Y, N, bias, "accel_run_epilogue", static_cast<hipStream_t>(stream))) return rc;
     if (flags & ~ACCEL_EPILOGUE_RELU) { set_error("accel_run_epilogue: unknown flags %d", flags); return ACCEL_ERR_ARG; }
-    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, bias,
+    return spmm_launch(h, X, Y, N, static_cast<hipStream_t>(stream), nullptr, nullptr, bias,
                        (flags & ACCEL_EPILOGUE_RELU) ? 1 : 0);
 }
 
@@ -711,30 +901,33 @@ int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup,
 {
     clear_error();
     if (warmup < 0 || iters < 0) { set_error("accel_time: bad warmup/iters"); return ACCEL_ERR_ARG; }
-    if (int rc = check_run(h, X, Y, N, nullptr, "accel_time")) return rc;
+    if (int rc = check_run(h, X, Y, N, nullptr, "accel_time", static_cast<hipStream_t>(stream))) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     for (int i = 0; i < warmup; i++)
-        if (int rc = spmm_launch(h, X, Y, N, s, nullptr)) return rc;
+        if (int rc = spmm_launch(h, X, Y, N, s)) return rc;
     ACCEL_HIP(hipStreamSynchronize(s));
     if (iters == 0) return ACCEL_OK;
-    // all launches are queued back to back; the events are read after one final wait
-    std::vector<hipEvent_t> ev((size_t)iters * 3, nullptr);
+    // All launches are queued back to back; the events are read after one final wait.  Per
+    // run: two events recorded around it, and two bound to the gather kernel itself (its
+    // start and its end: these put nothing between the run's kernels).
+    std::vector<hipEvent_t> ev((size_t)iters * 4, nullptr);
     int rc = ACCEL_OK;
     for (auto &e : ev)
         if (hipEventCreate(&e) != hipSuccess) { rc = ACCEL_ERR_HIP; set_error("hipEventCreate failed"); break; }
     for (int i = 0; i < iters && !rc; i++) {
-        hipError_t e = hipEventRecord(ev[3 * i], s);
-        if (e == hipSuccess) rc = spmm_launch(h, X, Y, N, s, ms_main ? ev[3 * i + 1] : nullptr);
-        if (!rc && e == hipSuccess) e = hipEventRecord(ev[3 * i + 2], s);
+        hipError_t e = hipEventRecord(ev[4 * i], s);
+        if (e == hipSuccess)
+            rc = spmm_launch(h, X, Y, N, s, ms_main ? ev[4 * i + 1] : nullptr, ms_main ? ev[4 * i + 2] : nullptr);
+        if (!rc && e == hipSuccess) e = hipEventRecord(ev[4 * i + 3], s);
         if (!rc && e != hipSuccess) { set_error("hipEventRecord: %s", hipGetErrorString(e)); rc = ACCEL_ERR_HIP; }
     }
     if (!rc && hipStreamSynchronize(s) != hipSuccess) { set_error("stream synchronisation failed"); rc = ACCEL_ERR_HIP; }
     for (int i = 0; i < iters && !rc; i++) {
         float t = 0.f;
-        hipError_t e = hipEventElapsedTime(&t, ev[3 * i], ev[3 * i + 2]);
+        hipError_t e = hipEventElapsedTime(&t, ev[4 * i], ev[4 * i + 3]);
         if (e == hipSuccess && ms_total) ms_total[i] = t;
         if (e == hipSuccess && ms_main) {
-            e = hipEventElapsedTime(&t, ev[3 * i], ev[3 * i + 1]);
+            e = hipEventElapsedTime(&t, ev[4 * i + 1], ev[4 * i + 2]);
             ms_main[i] = t;
         }
         if (e != hipSuccess) { set_error("event timing failed: %s", hipGetErrorString(e)); rc = ACCEL_ERR_HIP; }

@@ -15,6 +15,7 @@ constexpr int kDegBound = ACCEL_DEG_BOUND;            // non-zeros per block4 en
 constexpr int kSlices = ACCEL_SLICES_PER_BLOCK;       // slices per entry (metadata ABI)
 constexpr int kSliceNz = kDegBound / kSlices;         // 32
 constexpr int kXcds = 8;                              // accelerator dies, each with its own L2
+constexpr int kCusPerDie = 32;                        // compute units per die: 256 on the whole GPU
 constexpr int kWavesPerGroup = 4;                     // wavefronts (work units) per workgroup (1, 2, 8: within 2 %)
 
 constexpr int kMaxGroups = 64;                        // column groups of the launch plan (8..64)
@@ -91,7 +92,7 @@ struct accel_handle {
     int32_t *block4 = nullptr;        // [4*n_blocks]  the .block4 metadata (upstream ABI)
     // launch plan derived from block4 (see preprocess.hip, "work list")
     int32_t *work = nullptr;          // [4*n_units] one int4 per wavefront
-    int64_t n_units = 0;              // multiple of 4 * kXcds
+    int64_t n_units = 0;              // multiple of 4 * plan_queues
     int64_t n_long_units = 0;         // units that write a partial sum
     int32_t *long_slot = nullptr;     // [n_split_rows+1] partial-sum slots of each split row
     // plan granularity: rows with more than plan_split non-zeros are cut into pieces of at
@@ -104,6 +105,9 @@ struct accel_handle {
     int plan_groups = 0;              // 0: by row length (row_groups); 8..64: the same for all rows
     int plan_team_option = 0;         // 0: choose from the size of the matrix; 1: wavefront units; 2: workgroup units
     int plan_panel_option = 0;        // 0: choose; else the column-panel width of wide operands
+    int plan_queues_option = 0;       // 0: from the device's shape; 1 or 8
+    int plan_queues = accel::kXcds;   // interleaved queues of the launch plan: 8 (one per die), or 1
+    int device_cus = 0;               // compute units of the device the handle was created on
     bool plan_team = false;           // a unit is worked on by a whole workgroup (small matrices)
     bool local = false;               // most non-zeros lie near the diagonal (sampled)
     int64_t n_split_rows = 0;         // rows with more than plan_split non-zeros
@@ -116,27 +120,46 @@ struct accel_handle {
     // scratch for the partial sums of long-row segments: [n_long_blocks * N]
     float *partial = nullptr;
     size_t partial_floats = 0;
-    // which stream used `partial` last, and an event recorded behind that run
-    hipStream_t partial_stream = nullptr;
-    hipEvent_t partial_done = nullptr;
-    bool partial_in_use = false;
-    // dense operands already checked (address, bytes needed): see check_operand in capi.hip
-    struct Checked { const void *p = nullptr; size_t bytes = 0; } checked[4];
-    int checked_next = 0;
+    // sorted position -> position in the caller's arrays, built by the first value update
+    int32_t *src_pos = nullptr;
+    // Which streams use the handle's mutable device memory (see order_run / order_update in
+    // capi.hip).  Runs read the sorted values and, with split rows, write and read `partial`;
+    // a value update rewrites the sorted values.  A tracked run leaves an event, bound to its
+    // last kernel, in the slot of its stream; nothing is ever asked of a stream after the call
+    // that used it has returned (the caller may have destroyed it).
+    static constexpr int kMaxStreams = 4;
+    struct StreamSlot {
+        hipStream_t stream = nullptr;
+        hipEvent_t done = nullptr;           // bound to the last kernel of the last tracked run on `stream`
+        bool live = false;                   // a run has been queued there since the last value update
+    } slot[kMaxStreams];
+    int next_victim = 0;                     // slot reused when a fifth stream turns up
+    int partial_slot = -1;                   // slot of the last run that used `partial`
+    bool track_runs = false;                 // the values have been updated once: every run is tracked
+    hipStream_t writer = nullptr;            // stream of the last value update
+    bool writer_pending = false;             // ... which may still be running
+    hipEvent_t writer_done = nullptr;        // recorded behind it
 };
 
 namespace accel {
 // preprocess.hip
-int preprocess_device(accel_handle *h);
-int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s);
-int refresh_sorted_csr(accel_handle *h, bool values_only, hipStream_t s);
-int hash_words_device(const void *words_dev, int64_t n, uint64_t seed, uint64_t *out_dev, hipStream_t s);
+struct SavedOrder {               // a degree-sort order read from a saved state
+    bool identity;                // the rows were already in order: no permutation stored
+    const uint32_t *perm_dev;     // [rows] on the device otherwise
+};
+int preprocess_device(accel_handle *h, const SavedOrder *given = nullptr);
+int build_source_positions(accel_handle *h, hipStream_t s);
+int gather_values(accel_handle *h, const float *val, hipStream_t s);
 // capi.hip
 void release_products(accel_handle *h);
+bool stream_is_capturing(hipStream_t s);
+int order_run(accel_handle *h, hipStream_t s, bool uses_partial, bool capturing, hipEvent_t *run_done);
+int order_update(accel_handle *h, hipStream_t s, bool capturing);
+int note_update(accel_handle *h, hipStream_t s, bool capturing);
 // spmm.hip
 int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
-                hipEvent_t after_main, const float *bias = nullptr, int relu = 0,
-                bool static_partial = false, int ld = 0);
+                hipEvent_t main_start = nullptr, hipEvent_t main_stop = nullptr, const float *bias = nullptr,
+                int relu = 0, bool static_partial = false, int ld = 0);
 int reserve_partial(accel_handle *h, size_t floats);
 int fill_u32(void *dst, uint32_t v, size_t n, hipStream_t s);
 int copy_u32(void *dst, const void *src, size_t n, hipStream_t s);

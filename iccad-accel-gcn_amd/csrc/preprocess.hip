@@ -508,7 +508,7 @@ __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
     const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
     const float *__restrict__ val, const int32_t *__restrict__ perm,
     const int32_t *__restrict__ s_indptr, const int *__restrict__ tile_first, int64_t last_row,
-    int64_t n_take, int32_t *__restrict__ s_idx, float *__restrict__ s_val)
+    int64_t n_take, int32_t *__restrict__ s_idx, float *__restrict__ s_val, int32_t *__restrict__ src_pos)
 {
     __shared__ int row_end[kPermuteTile + 1];        // s_indptr[first + j + 1]
     __shared__ int64_t shift[kPermuteTile + 1];      // source position minus sorted position, per row
@@ -533,8 +533,9 @@ __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
             if ((int64_t)row_end[mid] > p) hi = mid; else lo = mid + 1;
         }
         const int64_t src = p + shift[lo];
-        if (s_idx) s_idx[p] = idx[src];              // null: only the values are gathered
-        s_val[p] = val[src];
+        if (s_idx) s_idx[p] = idx[src];
+        if (s_val) s_val[p] = val[src];
+        if (src_pos) src_pos[p] = (int32_t)src;      // where the non-zero sits in the caller's arrays
     }
 }
 
@@ -543,8 +544,9 @@ __global__ __launch_bounds__(kThreads) void permute_csr_kernel(
 // col_group(column, row_groups(degree)), stably inside each group, so that a
 // work unit of such a row touches rows of X that belong to one column group.
 // One workgroup per split row; counts[lr*64 + g] receives the size of each group
-// (counts may be null).  With s_idx null only the values are written (the columns of the
-// sorted copy are in place already and only the values changed).
+// (counts may be null).  Each of the three outputs may be null: the columns, the values,
+// and src_pos, the position of each non-zero in the caller's arrays (what a later value
+// update gathers through).
 // ---------------------------------------------------------------------------
 constexpr int kGroupRound = 4;   // elements per thread between two barriers of group_long_rows_kernel
 
@@ -552,7 +554,8 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
     const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
     const float *__restrict__ val, const int32_t *__restrict__ perm,
     const int32_t *__restrict__ s_indptr, int64_t first_long_row, int forced_groups,
-    int32_t *__restrict__ s_idx, float *__restrict__ s_val, int *__restrict__ counts)
+    int32_t *__restrict__ s_idx, float *__restrict__ s_val, int *__restrict__ counts,
+    int32_t *__restrict__ src_pos)
 {
     __shared__ int cnt[kMaxGroups];
     __shared__ int base[kMaxGroups];
@@ -589,7 +592,7 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
             const int i = c0 + e * kThreads + (int)threadIdx.x;
             valid[e] = i < d;
             col[e] = valid[e] ? idx[src0 + i] : 0;
-            v[e] = valid[e] ? val[src0 + i] : 0.0f;
+            v[e] = valid[e] && s_val ? val[src0 + i] : 0.0f;
             g[e] = col_group(col[e], ng);
             wave_cnt[flip][e][w][lane] = 0;             // each wavefront clears its own rows
         }
@@ -615,7 +618,8 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_kernel(
                 for (int q = 0; q < kThreads / 64; q++) pos += wave_cnt[flip][e2][q][g[e]];
             for (int q = 0; q < w; q++) pos += wave_cnt[flip][e][q][g[e]];
             if (s_idx) s_idx[dst0 + pos] = col[e];
-            s_val[dst0 + pos] = v[e];
+            if (s_val) s_val[dst0 + pos] = v[e];
+            if (src_pos) src_pos[dst0 + pos] = (int32_t)(src0 + c0 + e * kThreads + (int)threadIdx.x);
         }
         __syncthreads();
         if ((int)threadIdx.x < kMaxGroups) {
@@ -639,7 +643,8 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_wave_kernel(
     const int32_t *__restrict__ indptr, const int32_t *__restrict__ idx,
     const float *__restrict__ val, const int32_t *__restrict__ perm,
     const int32_t *__restrict__ s_indptr, int64_t first_long_row, int n_rows, int forced_groups,
-    int32_t *__restrict__ s_idx, float *__restrict__ s_val, int *__restrict__ counts)
+    int32_t *__restrict__ s_idx, float *__restrict__ s_val, int *__restrict__ counts,
+    int32_t *__restrict__ src_pos)
 {
     static_assert(kMaxGroups == 64, "one lane per column group");
     __shared__ int cnt[kThreads / 64][kMaxGroups];
@@ -671,7 +676,7 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_wave_kernel(
         const int i = c0 + lane;
         const bool valid = i < d;
         const int col = valid ? idx[src0 + i] : 0;
-        const float v = valid ? val[src0 + i] : 0.0f;
+        const float v = valid && s_val ? val[src0 + i] : 0.0f;
         const int g = col_group(col, ng);
         unsigned long long peers = __ballot(valid);      // lanes with the same group
 #pragma unroll
@@ -686,7 +691,8 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_wave_kernel(
         __builtin_amdgcn_wave_barrier();
         if (valid) {
             if (s_idx) s_idx[dst0 + pos] = col;
-            s_val[dst0 + pos] = v;
+            if (s_val) s_val[dst0 + pos] = v;
+            if (src_pos) src_pos[dst0 + pos] = (int32_t)(src0 + i);
             if (rank == 0) my[g] += __popcll(peers);     // one lane per group present
         }
         __builtin_amdgcn_wave_barrier();
@@ -698,12 +704,12 @@ __global__ __launch_bounds__(kThreads) void group_long_rows_wave_kernel(
 static void launch_permute_csr(const int32_t *indptr, const int32_t *idx, const float *val,
                                const int32_t *perm, const int32_t *s_indptr, int64_t rows,
                                int64_t first_long, int64_t n_take, int *tile_first, int32_t *s_idx,
-                               float *s_val, hipStream_t s)
+                               float *s_val, int32_t *src_pos, hipStream_t s)
 {
     if (n_take <= 0) return;
     tile_first_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(s_indptr, rows, n_take, tile_first);
     permute_csr_kernel<<<dim3((unsigned)((n_take + kPermuteTile - 1) / kPermuteTile)), dim3(kThreads), 0, s>>>(
-        indptr, idx, val, perm, s_indptr, tile_first, first_long - 1, n_take, s_idx, s_val);
+        indptr, idx, val, perm, s_indptr, tile_first, first_long - 1, n_take, s_idx, s_val, src_pos);
 }
 
 // Regroups the n_long split rows (the last rows of the sorted order, ascending by
@@ -711,17 +717,18 @@ static void launch_permute_csr(const int32_t *indptr, const int32_t *idx, const 
 static void launch_group_long_rows(const int32_t *indptr, const int32_t *idx, const float *val,
                                    const int32_t *perm, const int32_t *s_indptr, int64_t first_long,
                                    int64_t n_long, int64_t n_wide, int forced_groups, int32_t *s_idx,
-                                   float *s_val, int *counts, hipStream_t s)
+                                   float *s_val, int *counts, int32_t *src_pos, hipStream_t s)
 {
     const int64_t n_narrow = n_long - n_wide;
     if (n_narrow > 0)
         group_long_rows_wave_kernel<<<dim3((unsigned)((n_narrow + kThreads / 64 - 1) / (kThreads / 64))),
                                       dim3(kThreads), 0, s>>>(
-            indptr, idx, val, perm, s_indptr, first_long, (int)n_narrow, forced_groups, s_idx, s_val, counts);
+            indptr, idx, val, perm, s_indptr, first_long, (int)n_narrow, forced_groups, s_idx, s_val, counts,
+            src_pos);
     if (n_wide > 0)
         group_long_rows_kernel<<<dim3((unsigned)n_wide), dim3(kThreads), 0, s>>>(
             indptr, idx, val, perm, s_indptr, first_long + n_narrow, forced_groups, s_idx, s_val,
-            counts ? counts + n_narrow * kMaxGroups : nullptr);
+            counts ? counts + n_narrow * kMaxGroups : nullptr, src_pos);
 }
 
 // ---------------------------------------------------------------------------
@@ -791,10 +798,10 @@ struct BinOffsets {
     int off[kPlanBins];      // where the pieces of a (row class, column group) bin start in their queue
 };
 
-__device__ __forceinline__ int64_t plan_index(int queue, int pos)
+__device__ __forceinline__ int64_t plan_index(int queue, int pos, int n_queues)
 {
-    // queue q, position p  ->  slot of wavefront (p % 4) in workgroup (p / 4) * 8 + q
-    return ((int64_t)(pos / kWavesPerGroup) * kXcds + queue) * kWavesPerGroup + pos % kWavesPerGroup;
+    // queue q, position p  ->  slot of wavefront (p % 4) in workgroup (p / 4) * n_queues + q
+    return ((int64_t)(pos / kWavesPerGroup) * n_queues + queue) * kWavesPerGroup + pos % kWavesPerGroup;
 }
 
 // The order of the split rows inside their (class, group) bins: key[lr] = the caller's row id
@@ -854,7 +861,7 @@ __global__ void plan_totals_kernel(const int *__restrict__ grp_pos, int n_long, 
 __global__ __launch_bounds__(kThreads) void emit_long_units_kernel(
     const int *__restrict__ gcount, const int32_t *__restrict__ s_indptr, int64_t first_long,
     const int *__restrict__ slot, const int *__restrict__ grp_pos, int n_long, int forced_groups,
-    int piece, const int *__restrict__ rank, BinOffsets bo, int4 *__restrict__ work)
+    int piece, const int *__restrict__ rank, BinOffsets bo, int n_queues, int4 *__restrict__ work)
 {
     const int t = blockIdx.x * kThreads + threadIdx.x;
     if (t >= n_long * kMaxGroups) return;
@@ -876,7 +883,7 @@ __global__ __launch_bounds__(kThreads) void emit_long_units_kernel(
                      grp_pos[(int64_t)bin * n_long];
     const int sl = slot[lr] + u_before;
     for (int k = 0, off = 0; off < c; k++, off += piece)
-        work[plan_index(g % kXcds, pos0 + k)] =
+        work[plan_index(g % n_queues, pos0 + k, n_queues)] =
             make_int4(kDegBound + 1 + sl + k, row, loc + off, min(piece, c - off));
 }
 
@@ -933,11 +940,13 @@ __global__ __launch_bounds__(kThreads) void short_unit_cost_kernel(
     heavy[sidx] = u.x * n_rows > light_nz;
 }
 
-// Non-zeros and pieces of the split rows per queue (column group g belongs to queue g % 8).
-// Thread t looks at (row t / 64, group t % 64), so lane l of a wavefront always holds a
-// group of queue l % 8: the wavefront's eight sums are formed with shuffles.
+// Non-zeros and pieces of the split rows per queue (column group g belongs to queue
+// g % n_queues, n_queues = 8 or 1).  Thread t looks at (row t / 64, group t % 64), so lane l
+// of a wavefront always holds a group with g % 8 == l % 8: the wavefront's eight sums are
+// formed with shuffles.
 __global__ __launch_bounds__(kThreads) void long_queue_load_kernel(
-    const int *__restrict__ gcount, int n_long, int piece, int shift, int *__restrict__ queue_cost)
+    const int *__restrict__ gcount, int n_long, int piece, int shift, int n_queues,
+    int *__restrict__ queue_cost)
 {
     static_assert(kMaxGroups == 64, "one wavefront per split row");
     const int64_t n = (int64_t)n_long * kMaxGroups;
@@ -953,7 +962,7 @@ __global__ __launch_bounds__(kThreads) void long_queue_load_kernel(
     v += __shfl_xor(v, 16);
     v += __shfl_xor(v, 32);
     const int lane = threadIdx.x & 63;
-    if (lane < kXcds && v) atomicAdd(&queue_cost[lane], v);
+    if (lane < kXcds && v) atomicAdd(&queue_cost[lane % n_queues], v);
 }
 
 struct QueueCuts {
@@ -972,27 +981,27 @@ __device__ __forceinline__ int queue_of(int running_cost, const QueueCuts &qc)
 // of the whole-row units' cost, level being the smallest common level that takes all of it.
 // One thread; total_cost points at the sum of the units' costs.
 __global__ void queue_cuts_kernel(const int *__restrict__ long_cost, const int *__restrict__ total_cost,
-                                  QueueCuts *__restrict__ out)
+                                  int n_queues, QueueCuts *__restrict__ out)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
     const long long short_cost = *total_cost;
     long long lc[kXcds], lo = 0, hi = short_cost;
-    for (int q = 0; q < kXcds; q++) {
+    for (int q = 0; q < n_queues; q++) {
         lc[q] = long_cost ? long_cost[q] : 0;
         if (lc[q] + short_cost > hi) hi = lc[q] + short_cost;
     }
     while (lo < hi) {                                  // smallest level that takes all of it
         const long long mid = (lo + hi) / 2;
         long long taken = 0;
-        for (int q = 0; q < kXcds; q++) taken += mid > lc[q] ? mid - lc[q] : 0;
+        for (int q = 0; q < n_queues; q++) taken += mid > lc[q] ? mid - lc[q] : 0;
         if (taken >= short_cost) hi = mid; else lo = mid + 1;
     }
     long long run = 0;
-    for (int q = 0; q < kXcds; q++) {
+    for (int q = 0; q < n_queues; q++) {
         out->cut[q] = (int)(run < short_cost ? run : short_cost);
         run += lo > lc[q] ? lo - lc[q] : 0;
     }
-    out->cut[kXcds] = INT_MAX;
+    for (int q = n_queues; q <= kXcds; q++) out->cut[q] = INT_MAX;   // queues that do not exist take nothing
 }
 
 // first[q] = rank of the first unit of queue q (n for queues that get none); first must hold n on entry.
@@ -1018,7 +1027,7 @@ constexpr int kTailLight = 2048;             // two rounds of the 1,024 wavefron
 __global__ __launch_bounds__(kThreads) void place_short_units_kernel(
     const int4 *__restrict__ units, const uint32_t *__restrict__ order, const int *__restrict__ running,
     const int *__restrict__ heavy_before, int n, const QueueCuts *__restrict__ cuts,
-    const int *__restrict__ first, PlanParams pp, int4 *__restrict__ work)
+    const int *__restrict__ first, PlanParams pp, int n_queues, int4 *__restrict__ work)
 {
     const int sidx = blockIdx.x * kThreads + threadIdx.x;
     if (sidx >= n) return;
@@ -1035,7 +1044,7 @@ __global__ __launch_bounds__(kThreads) void place_short_units_kernel(
         pos = n_q - (light_all - light_me);                                // held back: the last ones
     else
         pos = (sidx - f) - max(0, light_me - kept);                        // in line, minus those held back before it
-    work[plan_index(q, pp.queue_long[q] + pos)] = units[order[sidx]];
+    work[plan_index(q, pp.queue_long[q] + pos, n_queues)] = units[order[sidx]];
 }
 
 }  // namespace
@@ -1150,6 +1159,7 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
     const int64_t n_long = h->n_split_rows;
     // pieces of split rows hold up to piece_nz non-zeros, units of several whole rows up to unit_nz
     const int unit_nz = h->plan_unit, piece_nz = std::max(h->plan_unit, h->plan_split), forced = h->plan_groups;
+    const int nq = h->plan_queues;                     // 8 interleaved queues, or 1 (plain order)
     DevBuf row_units(tmp), grp_units(tmp), sums(tmp), totals(tmp), dslot, scnt(tmp), qload(tmp), lkey(tmp),
         lrank(tmp);
     int rc;
@@ -1186,7 +1196,7 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
             gcount, s_indptr, first_long, (int)n_long, forced, piece_nz, lrank.as<int>(),
             row_units.as<int>(), grp_units.as<int>());
         long_queue_load_kernel<<<dim3(std::min(grid_for(n_long * kMaxGroups), 1024u)), dim3(kThreads), 0, s>>>(
-            gcount, (int)n_long, piece_nz, cost_shift, qload.as<int>());
+            gcount, (int)n_long, piece_nz, cost_shift, nq, qload.as<int>());
         if ((rc = device_scan<SumOp, false>(row_units.as<int>(), n_long, dslot.as<int>(),
                                             dslot.as<int>() + n_long, sums.as<int>(), s)))
             return rc;
@@ -1252,7 +1262,7 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
                                             csums.as<int>(), s)))
             return rc;
         queue_cuts_kernel<<<dim3(1), dim3(1), 0, s>>>(n_long > 0 ? qload.as<int>() : nullptr, cost.as<int>() + n,
-                                                      cuts.as<QueueCuts>());
+                                                      nq, cuts.as<QueueCuts>());
         if ((rc = fill_u32(first.p, (uint32_t)n, kXcds + 1, s))) return rc;
         queue_first_kernel<<<dim3(grid_for(n)), dim3(kThreads), 0, s>>>(cost.as<int>(), n, cuts.as<QueueCuts>(),
                                                                        first.as<int>());
@@ -1279,15 +1289,15 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
         for (int ng = kMaxGroups; ng >= kXcds; ng /= 2)
             for (int g = 0; g < ng; g++) {
                 const int b = plan_bin(ng, g);
-                bo.off[b] = pp.queue_long[g % kXcds];
-                pp.queue_long[g % kXcds] += tot[b + 1] - tot[b];
+                bo.off[b] = pp.queue_long[g % nq];
+                pp.queue_long[g % nq] += tot[b + 1] - tot[b];
             }
     const int64_t n_long_units = n_long > 0 ? tot[kPlanBins] : 0;
     int64_t per_queue = 0;
-    for (int q = 0; q < kXcds; q++)
+    for (int q = 0; q < nq; q++)
         per_queue = std::max<int64_t>(per_queue, (int64_t)pp.queue_long[q] + (first_h[q + 1] - first_h[q]));
     per_queue = (per_queue + kWavesPerGroup - 1) / kWavesPerGroup * kWavesPerGroup;
-    const int64_t n_units = per_queue * kXcds;
+    const int64_t n_units = per_queue * nq;
     if (n_units > (int64_t)INT_MAX) {
         set_error("the launch plan would exceed 2^31 work units");
         return ACCEL_ERR_ARG;
@@ -1298,11 +1308,11 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
     if (n_long > 0)
         emit_long_units_kernel<<<dim3(grid_for(n_long * kMaxGroups)), dim3(kThreads), 0, s>>>(
             gcount, s_indptr, first_long, dslot.as<int>(), grp_units.as<int>(), (int)n_long, forced,
-            piece_nz, lrank.as<int>(), bo, dwork.as<int4>());
+            piece_nz, lrank.as<int>(), bo, nq, dwork.as<int4>());
     if (n_short_units > 0)
         place_short_units_kernel<<<dim3(grid_for(n_short_units)), dim3(kThreads), 0, s>>>(
             units.as<int4>(), order, cost.as<int>(), heavy.as<int>(), (int)n_short_units, cuts.as<QueueCuts>(),
-            first.as<int>(), pp, dwork.as<int4>());
+            first.as<int>(), pp, nq, dwork.as<int4>());
     ACCEL_HIP(hipGetLastError());
     ACCEL_HIP(hipStreamSynchronize(s));
     h->n_units = n_units;
@@ -1362,99 +1372,92 @@ static int choose_plan_split(int64_t rows, int64_t nnz, bool team)
     return team ? kDegBound : kPlanSplit;        // workgroup units: rows up to one unit stay whole
 }
 
-// 64-bit content hash of n 4-byte words: the sum over i of mix(i, word i) modulo 2^64,
-// so the order of the additions does not matter.  *out must be zero on entry.
-__device__ __forceinline__ uint64_t mix64(uint64_t x)
+// New values on an unchanged structure reach the sorted copy through a map from sorted
+// position to the position in the caller's arrays.  The map is what the regathering kernels
+// of the preprocessing compute anyway (where each non-zero comes from); it is built here, by
+// those kernels with only that output switched on, the first time a handle's values are
+// replaced, and kept.  Needs perm (or identity_perm), s_indptr, nnz_short, n_split_rows,
+// n_wide_rows and plan_groups as the preprocessing left them.  Allocates; synchronises s.
+int build_source_positions(accel_handle *h, hipStream_t s)
 {
-    x += 0x9E3779B97F4A7C15ull;
-    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
-    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
-    return x ^ (x >> 31);
-}
-
-__global__ __launch_bounds__(kThreads) void hash_words_kernel(const uint32_t *__restrict__ a, int64_t n,
-                                                              uint64_t seed,
-                                                              unsigned long long *__restrict__ out)
-{
-    __shared__ unsigned long long part[kThreads / 64];
-    uint64_t acc = 0;
-    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads)
-        acc += mix64((((uint64_t)i << 32) | a[i]) ^ seed);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor((unsigned long long)acc, off);
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int q = 1; q < kThreads / 64; q++) acc += part[q];
-        atomicAdd(out, (unsigned long long)acc);
-    }
-}
-
-int hash_words_device(const void *words_dev, int64_t n, uint64_t seed, uint64_t *out_dev, hipStream_t s)
-{
-    if (n <= 0) return ACCEL_OK;
-    const unsigned g = (unsigned)std::min<int64_t>((n + kThreads - 1) / kThreads, 4096);
-    hash_words_kernel<<<dim3(g), dim3(kThreads), 0, s>>>(static_cast<const uint32_t *>(words_dev), n, seed,
-                                                         reinterpret_cast<unsigned long long *>(out_dev));
-    ACCEL_HIP(hipGetLastError());
-    return ACCEL_OK;
-}
-
-// The non-zeros of the caller's CSR gathered into the degree-sorted copy the handle owns
-// (s_idx, s_val), in place: rows that stay whole keep the order of their non-zeros, split rows
-// are regrouped by column group.  Needs perm (or identity_perm), s_indptr, nnz_short,
-// n_split_rows, n_wide_rows and plan_groups.  This is also how new values on an unchanged
-// structure reach the copy the kernels read (values_only: the columns are left as they are).
-int refresh_sorted_csr(accel_handle *h, bool values_only, hipStream_t s)
-{
-    if (!h->owns_sorted) {                  // the sorted copy is the caller's CSR itself
-        h->s_idx = h->idx;
-        h->s_val = h->val;
-        return ACCEL_OK;
-    }
+    if (h->src_pos || !h->owns_sorted || h->nnz == 0) return ACCEL_OK;
     const int64_t rows = h->rows, n_long = h->n_split_rows, first_long = rows - n_long;
     const int64_t nnz_short = h->nnz_short;
-    int32_t *sidx = values_only ? nullptr : const_cast<int32_t *>(h->s_idx);
-    float *sval = const_cast<float *>(h->s_val);
-    DevBuf tiles;
+    DevBuf map, tiles;
+    if (int rc = map.alloc(sizeof(int32_t) * (size_t)h->nnz)) return rc;
     if (nnz_short > 0) {
-        if (h->identity_perm) {
-            if (sidx)
-                ACCEL_HIP(hipMemcpyAsync(sidx, h->idx, sizeof(int32_t) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
-            ACCEL_HIP(hipMemcpyAsync(sval, h->val, sizeof(float) * (size_t)nnz_short, hipMemcpyDeviceToDevice, s));
-        } else {
-            if (int rc = tiles.alloc(sizeof(int) * (size_t)(nnz_short / kPermuteTile + 2))) return rc;
-            launch_permute_csr(h->indptr, h->idx, h->val, h->perm, h->s_indptr, rows, first_long, nnz_short,
-                               tiles.as<int>(), sidx, sval, s);
-        }
+        if (int rc = tiles.alloc(sizeof(int) * (size_t)(nnz_short / kPermuteTile + 2))) return rc;
+        launch_permute_csr(h->indptr, h->idx, h->val, h->perm, h->s_indptr, rows, first_long, nnz_short,
+                           tiles.as<int>(), nullptr, nullptr, map.as<int32_t>(), s);
     }
     if (n_long > 0)
         launch_group_long_rows(h->indptr, h->idx, h->val, h->perm, h->s_indptr, first_long, n_long,
-                               std::min<int64_t>(h->n_wide_rows, n_long), h->plan_groups, sidx, sval, nullptr, s);
+                               std::min<int64_t>(h->n_wide_rows, n_long), h->plan_groups, nullptr, nullptr,
+                               nullptr, map.as<int32_t>(), s);
     ACCEL_HIP(hipGetLastError());
     ACCEL_HIP(hipStreamSynchronize(s));     // `tiles` is released on return
+    h->src_pos = static_cast<int32_t *>(map.release());
     return ACCEL_OK;
 }
 
-// The degree-sorted copy of the CSR for products that come from a saved state (perm,
-// s_indptr, the plan): allocates it and fills it as above.  nnz_short = non-zeros of the
-// rows that are not split.
-int rebuild_sorted_csr(accel_handle *h, int64_t nnz_short, hipStream_t s)
+// s_val[p] = val[src_pos[p]]: four non-zeros per thread, the map read and the values written
+// as 16-byte vectors (both arrays come from hipMalloc and start 256-byte aligned).
+__global__ __launch_bounds__(kThreads) void gather_values_kernel(const float *__restrict__ val,
+                                                                 const int32_t *__restrict__ src_pos,
+                                                                 float *__restrict__ s_val, int64_t nnz)
 {
-    h->nnz_short = nnz_short;
-    h->owns_sorted = !(h->identity_perm && h->n_split_rows == 0);
-    if (h->owns_sorted) {
-        DevBuf sidx, sval;
-        int rc;
-        if ((rc = sidx.alloc(sizeof(int32_t) * (size_t)h->nnz))) { h->owns_sorted = false; return rc; }
-        if ((rc = sval.alloc(sizeof(float) * (size_t)h->nnz))) { h->owns_sorted = false; return rc; }
-        h->s_idx = static_cast<int32_t *>(sidx.release());
-        h->s_val = static_cast<float *>(sval.release());
+    const int64_t p = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 4;
+    if (p + 4 <= nnz) {
+        const int4 q = *reinterpret_cast<const int4 *>(src_pos + p);
+        const float4 v = make_float4(val[q.x], val[q.y], val[q.z], val[q.w]);
+        *reinterpret_cast<float4 *>(s_val + p) = v;
+    } else {
+        for (int64_t i = p; i < nnz; i++) s_val[i] = val[src_pos[i]];
     }
-    return refresh_sorted_csr(h, false, s); // on failure release_products frees what was allocated
 }
 
-int preprocess_device(accel_handle *h)
+// One launch on s, no allocation, no wait: the sorted copy of the values from `val` (nnz
+// floats in the caller's order).  The map must exist.
+int gather_values(accel_handle *h, const float *val, hipStream_t s)
+{
+    if (!h->owns_sorted || h->nnz == 0) return ACCEL_OK;
+    if (!h->src_pos) {
+        set_error("internal: the position map of the value update is missing");
+        return ACCEL_ERR_STATE;
+    }
+    const int64_t threads = (h->nnz + 3) / 4;
+    gather_values_kernel<<<dim3(grid_for(threads)), dim3(kThreads), 0, s>>>(
+        val, h->src_pos, const_cast<float *>(h->s_val), h->nnz);
+    ACCEL_HIP(hipGetLastError());
+    return ACCEL_OK;
+}
+
+// A row order that comes from a saved state is taken only if it is the order the sort would
+// produce: ascending degree, ties by ascending row id.  That order is unique, so checking
+// that the pairs (degree, row) strictly increase along it and that every entry is a row
+// index proves it (strictly increasing pairs cannot repeat a row, and rows of them are then
+// all the rows).  Also writes the degrees in that order.
+__global__ __launch_bounds__(kThreads) void check_given_order_kernel(const uint32_t *__restrict__ deg,
+                                                                     const uint32_t *__restrict__ perm,
+                                                                     int64_t rows, uint32_t *__restrict__ sdeg,
+                                                                     int *__restrict__ bad)
+{
+    const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= rows) return;
+    const uint32_t p = perm[i];
+    if (p >= (uint64_t)rows) { *bad = 1; sdeg[i] = 0; return; }
+    const uint32_t d = deg[p];
+    sdeg[i] = d;
+    if (i > 0) {
+        const uint32_t q = perm[i - 1];
+        if (q >= (uint64_t)rows) { *bad = 1; return; }
+        const uint32_t dq = deg[q];
+        if (dq > d || (dq == d && q >= p)) *bad = 1;
+    }
+}
+
+// given: a row order from a saved state (checked before it is used), or null to sort.
+int preprocess_device(accel_handle *h, const SavedOrder *given)
 {
     const auto t0 = std::chrono::steady_clock::now();
     hipStream_t s = nullptr;
@@ -1472,6 +1475,11 @@ int preprocess_device(accel_handle *h)
     // a wavefront never takes more than plan_unit non-zeros; a workgroup takes a whole row of
     // up to plan_split even when units of several rows are kept smaller
     if (!h->plan_team) h->plan_split = std::min(h->plan_split, h->plan_unit);
+    // Eight interleaved queues when the device is the whole MI355X (8 dies of 32 compute
+    // units, workgroup i on die i % 8); any other shape (a partition of the GPU) gets the
+    // plan in plain order, one queue, whose column groups are still worked on one by one.
+    h->plan_queues = h->plan_queues_option > 0 ? h->plan_queues_option
+                                               : (h->device_cus == kXcds * kCusPerDie ? kXcds : 1);
     if (rows == 0) {
         h->identity_perm = true;
         h->ready = true;
@@ -1537,7 +1545,28 @@ int preprocess_device(accel_handle *h)
     // ---- degree sort ------------------------------------------------------
     uint32_t *sdeg = deg.as<uint32_t>();
     uint32_t *perm = nullptr;
-    if (!h->identity_perm) {
+    DevBuf given_deg(&tmp), given_bad(&tmp);
+    if (given && given->identity != h->identity_perm) {
+        set_error("the saved state was made for rows in another order (it says the rows are %s sorted by "
+                  "degree, this CSR's are%s)", given->identity ? "already" : "not", h->identity_perm ? "" : " not");
+        return ACCEL_ERR_META;
+    }
+    if (!h->identity_perm && given) {
+        if ((rc = given_deg.alloc(sizeof(uint32_t) * (size_t)rows))) return rc;
+        if ((rc = given_bad.alloc(sizeof(int)))) return rc;
+        ACCEL_HIP(hipMemsetAsync(given_bad.p, 0, sizeof(int), s));
+        check_given_order_kernel<<<dim3(grid_for(rows)), dim3(kThreads), 0, s>>>(
+            deg.as<uint32_t>(), given->perm_dev, rows, given_deg.as<uint32_t>(), given_bad.as<int>());
+        int bad = 0;
+        ACCEL_HIP(hipMemcpyAsync(&bad, given_bad.p, sizeof(int), hipMemcpyDeviceToHost, s));
+        ACCEL_HIP(hipStreamSynchronize(s));
+        if (bad) {
+            set_error("the saved row order is not the degree order of this CSR (state of another matrix, or damaged)");
+            return ACCEL_ERR_META;
+        }
+        sdeg = given_deg.as<uint32_t>();
+        perm = const_cast<uint32_t *>(given->perm_dev);
+    } else if (!h->identity_perm) {
         // unsorted input has max_degree >= 1, so at least one pass runs
         if ((rc = radix_sort_pairs(&tmp, deg.as<uint32_t>(), rows, (uint32_t)hs.max_degree, s, &sdeg, &perm)))
             return rc;
@@ -1617,7 +1646,7 @@ int preprocess_device(accel_handle *h)
             if (nnz_short > 0) {
                 if ((rc = tiles.alloc(sizeof(int) * (size_t)(nnz_short / kPermuteTile + 2)))) return rc;
                 launch_permute_csr(h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), rows, first_long, nnz_short,
-                                   tiles.as<int>(), sidx.as<int32_t>(), sval.as<float>(), s);
+                                   tiles.as<int>(), sidx.as<int32_t>(), sval.as<float>(), nullptr, s);
             }
             ACCEL_HIP(hipMemcpyAsync(permbuf.p, perm, sizeof(int32_t) * (size_t)rows,
                                      hipMemcpyDeviceToDevice, s));
@@ -1626,7 +1655,7 @@ int preprocess_device(accel_handle *h)
             if ((rc = gcount.alloc(sizeof(int) * (size_t)n_long * kMaxGroups))) return rc;
             launch_group_long_rows(h->indptr, h->idx, h->val, pm, sip.as<int32_t>(), first_long, n_long,
                                    std::min<int64_t>(hs.n_wide_rows, n_long), h->plan_groups,
-                                   sidx.as<int32_t>(), sval.as<float>(), gcount.as<int>(), s);
+                                   sidx.as<int32_t>(), sval.as<float>(), gcount.as<int>(), nullptr, s);
         }
         ACCEL_HIP(hipGetLastError());
     }

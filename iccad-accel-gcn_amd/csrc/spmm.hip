@@ -30,6 +30,8 @@
 // workgroups of the same launch: Y = A X holds after every run with no memset.
 #include <mutex>
 
+#include <hip/hip_ext.h>
+
 #include "internal.h"
 
 // Partial sums for accel_run_static, the entry point that allocates nothing: one copy of
@@ -510,11 +512,25 @@ struct LaunchArgs {
     int N, ld, n_zero_rows, n_zero_groups;
     const float *bias;
     int relu;
+    // events bound to this launch itself (its start and its end), or null: unlike an event
+    // recorded behind the launch they put no packet of their own into the queue
+    hipEvent_t start_ev, stop_ev;
 };
 
 template <int L, int VEC, bool kWide, bool kShift>
 void launch_one(const LaunchArgs &a)
 {
+    if (a.start_ev || a.stop_ev) {
+        if (a.team)
+            hipExtLaunchKernelGGL((spmm_team_kernel<L, VEC, kWide, kShift>), a.grid, dim3(kWgThreads), 0, a.stream,
+                                  a.start_ev, a.stop_ev, 0, a.work, a.n_units, a.s_idx, a.s_val, a.perm, a.X, a.Y,
+                                  a.partial, a.N, a.ld, a.n_zero_rows, a.n_zero_groups, a.bias, a.relu);
+        else
+            hipExtLaunchKernelGGL((spmm_gather_kernel<L, VEC, kWide, kShift>), a.grid, dim3(kWgThreads), 0, a.stream,
+                                  a.start_ev, a.stop_ev, 0, a.work, a.n_units, a.s_idx, a.s_val, a.perm, a.X, a.Y,
+                                  a.partial, a.N, a.ld, a.n_zero_rows, a.n_zero_groups, a.bias, a.relu);
+        return;
+    }
     if (a.team)
         spmm_team_kernel<L, VEC, kWide, kShift><<<a.grid, dim3(kWgThreads), 0, a.stream>>>(
             a.work, a.n_units, a.s_idx, a.s_val, a.perm, a.X, a.Y, a.partial, a.N, a.ld, a.n_zero_rows,
@@ -607,7 +623,8 @@ static int static_scratch_address(float **out)
 int reserve_partial(accel_handle *h, size_t floats)
 {
     if (h->partial_floats >= floats) return ACCEL_OK;
-    if (h->partial_in_use) (void)hipEventSynchronize(h->partial_done);   // nobody reads the old one
+    if (h->partial_slot >= 0 && hipEventSynchronize(h->slot[h->partial_slot].done) != hipSuccess)
+        (void)hipGetLastError();                       // nobody reads the old one (hipFree waits for the device as well)
     if (h->partial) (void)hipFree(h->partial);
     h->partial = nullptr;
     h->partial_floats = 0;
@@ -620,10 +637,14 @@ int reserve_partial(accel_handle *h, size_t floats)
     return ACCEL_OK;
 }
 
+// main_start / main_stop: events bound to the gather kernel (to the first and the last launch
+// when the run is done in column panels), for timing it alone.
 int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t stream,
-                hipEvent_t after_main, const float *bias, int relu, bool static_partial, int ld)
+                hipEvent_t main_start, hipEvent_t main_stop, const float *bias, int relu, bool static_partial,
+                int ld)
 {
     if (h->rows == 0) return ACCEL_OK;
+    (void)hipGetLastError();                         // launch errors are read back below: start from a clean slate
     if (ld <= 0) ld = N;                             // rows of X and Y are ld floats apart
     // 16-byte vectors whenever a row holds one.  When N is not a multiple of 4, or X or Y
     // is not 16-byte aligned, rows start at odd multiples of 4 bytes: the vectors are then
@@ -637,7 +658,9 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     // partial sums of the pieces of split rows: the handle's buffer (allocated here when a
     // run needs more than it holds), or this GPU's static array, which is never allocated
     float *partial = h->partial;
-    bool guard_partial = false;
+    const bool uses_handle_partial = !static_partial && h->n_long_units > 0;
+    // the capture status is only needed where something depends on it
+    const bool capturing = (uses_handle_partial || h->writer_pending) && stream_is_capturing(stream);
     if (static_partial) {
         partial = nullptr;
         const size_t need = (size_t)h->n_long_units * (size_t)ld;
@@ -649,21 +672,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         }
         if (need > 0)
             if (int rc = static_scratch_address(&partial)) return rc;
-    } else if (h->n_long_units > 0) {
-        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        (void)hipStreamIsCapturing(stream, &cap);
-        if (hipGetLastError() != hipSuccess) cap = hipStreamCaptureStatusNone;
-        const bool capturing = cap != hipStreamCaptureStatusNone;
-        // The buffer is shared by all runs of this handle: a run on another stream may only
-        // start once the previous one has finished (runs queued on one stream are ordered).
-        if (h->partial_in_use && stream != h->partial_stream && !capturing &&
-            hipEventQuery(h->partial_done) == hipErrorNotReady) {
-            (void)hipGetLastError();
-            set_error("this handle is still running on another stream; its partial-sum buffer is "
-                      "shared: wait for that run, or use one handle per stream");
-            return ACCEL_ERR_STATE;
-        }
-        (void)hipGetLastError();
+    } else if (uses_handle_partial) {
         const size_t need = (size_t)h->n_long_units * (size_t)ld;
         if (h->partial_floats < need) {
             if (capturing) {
@@ -674,8 +683,13 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
             if (int rc = reserve_partial(h, need)) return rc;
         }
         partial = h->partial;
-        guard_partial = !capturing;
     }
+    // The buffer is shared by all runs of this handle, and a value update may still be
+    // rewriting what this run reads: a run on another stream than the one that used them
+    // last waits for that stream on the device (runs queued on one stream are ordered anyway).
+    hipEvent_t run_done = nullptr;                  // to be bound to the run's last kernel
+    if (int rc = order_run(h, stream, uses_handle_partial, capturing, &run_done)) return rc;
+    const bool has_reduce = h->n_split_rows > 0;
     // Wide operands are computed one column panel at a time (all units for the first
     // panel, then all units for the next): a panel's slice of X is what the L2s have
     // to hold, and a narrower slice means more rows of X fit.
@@ -698,10 +712,10 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         int L = 1;                                   // lanes per row: one per vector, a power of two
         while (L * vec < n && L < 64) L <<= 1;
         // zero-fill workgroups come first; their count is rounded up to a multiple of the
-        // die count so that entry group i still lands on die i % 8 (surplus ones exit at once)
+        // queue count so that entry group i still lands on die i % 8 (surplus ones exit at once)
         const int zr = zero_rows_per_group(n);
         int64_t zero_groups = (h->n_zero_rows + zr - 1) / zr;
-        zero_groups = (zero_groups + kXcds - 1) / kXcds * kXcds;
+        zero_groups = (zero_groups + h->plan_queues - 1) / h->plan_queues * h->plan_queues;
         const int64_t groups = entry_groups + zero_groups;
         if (groups > 0x7fffffffLL) {
             set_error("launch of %lld workgroups exceeds the grid limit", (long long)groups);
@@ -712,29 +726,35 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         const float *Xp = X ? X + c0 : X;
         float *Yp = Y + c0, *Pp = partial ? partial + c0 : nullptr;
         const float *bp = bias ? bias + c0 : nullptr;
+        const bool first = c0 == 0, last = c0 + panel >= N;
+        hipEvent_t stop = last ? main_stop : nullptr;
+        if (last && !stop && !has_reduce) stop = run_done;      // the run ends with this launch
         const LaunchArgs la{h->plan_team, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
-                            Xp, Yp, Pp, n, ld, (int)h->n_zero_rows, (int)zero_groups, bp, relu};
+                            Xp, Yp, Pp, n, ld, (int)h->n_zero_rows, (int)zero_groups, bp, relu,
+                            first ? main_start : nullptr, stop};
         const int rc = launch_for_mode(mode, wide, L, la);
         if (rc) return rc;
     }
-    if (after_main) ACCEL_HIP(hipEventRecord(after_main, stream));
-    if (h->n_split_rows > 0) {
+    if (!has_reduce && run_done && main_stop)       // the one launch cannot carry both events
+        ACCEL_HIP(hipEventRecord(run_done, stream));
+    if (has_reduce) {
         // one launch: rows with very many slots (the last n_big rows) get a workgroup each, the
         // others share one between 4, 2 or 1 rows depending on how many threads N can use
         const int n_split = (int)h->n_split_rows, n_big = (int)h->n_big_rows, n_shared = n_split - n_big;
         const int rpw = N <= 64 ? 4 : N <= 128 ? 2 : 1;
         const int shared_groups = (n_shared + rpw - 1) / rpw;
-        long_row_reduce_kernel<<<dim3((unsigned)(shared_groups + n_big)), dim3(kReduceThreads), 0, stream>>>(
-            partial, h->long_slot, h->perm, h->rows - h->n_split_rows, n_shared, shared_groups, rpw,
-            n_split, Y, N, ld, bias, relu);
+        const dim3 rgrid((unsigned)(shared_groups + n_big));
+        if (run_done)
+            hipExtLaunchKernelGGL(long_row_reduce_kernel, rgrid, dim3(kReduceThreads), 0, stream, nullptr, run_done,
+                                  0, (const float *)partial, (const int32_t *)h->long_slot, (const int32_t *)h->perm,
+                                  (int64_t)(h->rows - h->n_split_rows), n_shared, shared_groups, rpw, n_split, Y, N,
+                                  ld, bias, relu);
+        else
+            long_row_reduce_kernel<<<rgrid, dim3(kReduceThreads), 0, stream>>>(
+                partial, h->long_slot, h->perm, h->rows - h->n_split_rows, n_shared, shared_groups, rpw,
+                n_split, Y, N, ld, bias, relu);
     }
     ACCEL_HIP(hipGetLastError());
-    if (guard_partial) {
-        if (!h->partial_done) ACCEL_HIP(hipEventCreateWithFlags(&h->partial_done, hipEventDisableTiming));
-        ACCEL_HIP(hipEventRecord(h->partial_done, stream));
-        h->partial_stream = stream;
-        h->partial_in_use = true;
-    }
     return ACCEL_OK;
 }
 

@@ -15,8 +15,9 @@ bool SPMM_ACCEL::preprocess()
     if (h) {
         // Upstream's kernel reads val on every launch (spmm_accel.cu:75), so a caller that
         // rewrote the array between two do_test calls computes with the new values; the
-        // sorted copy this operator computes from is brought up to date the same way.
-        if (accel_update_values(h, val, ACCEL_PTR_DEVICE) != ACCEL_OK) {
+        // sorted copy this operator computes from is brought up to date by one kernel on
+        // the stream of the launches, with no wait on the host.
+        if (accel_update_values_async(h, val, nullptr) != ACCEL_OK) {
             err = accel_last_error();
             return false;
         }
@@ -25,11 +26,12 @@ bool SPMM_ACCEL::preprocess()
     err.clear();
     int rc = accel_create(ptr, idx, val, num_v, num_v, num_e, ACCEL_PTR_DEVICE, &h);
     if (!rc) {
-        // A state saved by an earlier run takes the place of the preprocessing, as upstream
-        // loads its metadata file instead of recomputing (spmm_accel.cu:122).  A state that
-        // is missing, damaged or belongs to another CSR is a stale cache entry, not an error.
+        // After set_save_state(true), a state saved by an earlier run takes the place of the
+        // sort, as upstream loads its metadata file instead of recomputing (spmm_accel.cu:122).
+        // A state that is missing, damaged or belongs to another CSR is a stale cache entry,
+        // not an error.
         const std::string state = meta_dir + _graph + ".accelstate";
-        from_state = accel_load_state(h, state.c_str()) == ACCEL_OK;
+        from_state = save_state && accel_load_state(h, state.c_str()) == ACCEL_OK;
         if (!from_state) {
             rc = accel_preprocess(h);
             if (!rc && save_state) (void)accel_save_state(h, state.c_str());   // best effort

@@ -5,11 +5,18 @@
 //   spmm_test                    time every <graphs>/*.config for dim 16..128 (main.cu:195-219)
 //   options: --graphs DIR (default ../graphs/)  --meta DIR (default ../block_level_meta/)
 //            --save-state   write <meta>/<graph>.accelstate after preprocessing; a later run
-//                           loads it instead of preprocessing (as upstream loads its .block4,
-//                           spmm_accel.cu:122) and says so on stderr
+//                           takes the row order from it instead of sorting (as upstream loads
+//                           its .block4, spmm_accel.cu:122) and says so on stderr
+//            --natural      read the graph in its own vertex order, <graph>.graph.ptrdump and
+//                           <graph>.graph.edgedump (the files upstream gives to its baselines,
+//                           main.cu:64-65), and hand that CSR to the operator, which sorts the
+//                           rows by degree itself and returns vout in the order given.  On graphs
+//                           whose numbering has locality this is the faster input: the launch plan
+//                           follows the caller's row ids, which the pre-sorted files have lost.
 //
-// Input files, as upstream reads them (main.cu:62-63, data.h:7-21): <graph>.new_indptr and
-// <graph>.new_indices, raw little-endian int32 (held in device memory here, not managed memory).  Values are all 1 and vin ~ U[0,1) from
+// Input files, as upstream reads them (main.cu:62-65, data.h:7-21): <graph>.new_indptr and
+// <graph>.new_indices (rows in ascending degree order), or the two .graph.* files with
+// --natural; raw little-endian int32 (held in device memory here, not managed memory).  Values are all 1 and vin ~ U[0,1) from
 // std::default_random_engine seeded with 123 (main.cu:90-93,114-121, value mode 3).
 // Output lines follow main.cu:40-49 and :161-167:
 //   err sum = <x>  validation pass!|fail!
@@ -34,6 +41,7 @@ std::string meta_dir = "../block_level_meta/";
 int dim_min = 16, dim_max = 128, interval = 1;
 int total_file_cnt = 0, current_file_cnt = 0;
 bool save_state = false;
+bool natural_order = false;
 
 // Upstream keeps every array in managed memory (data.h:15) and lets the pages migrate.
 // Here the arrays live in device memory and are copied explicitly: on a GPU that runs
@@ -106,10 +114,12 @@ int test_graph(const std::string &graph, int spec_dim, bool checking, bool timin
     if (spec_dim > 0) lo = hi = spec_dim;
 
     std::vector<int> h_ptr, h_idx;
-    if (!read_file(base_dir + graph + ".new_indptr", h_ptr)) return 1;
-    if (!read_file(base_dir + graph + ".new_indices", h_idx)) return 1;
+    const std::string ptr_file = graph + (natural_order ? ".graph.ptrdump" : ".new_indptr");
+    const std::string idx_file = graph + (natural_order ? ".graph.edgedump" : ".new_indices");
+    if (!read_file(base_dir + ptr_file, h_ptr)) return 1;
+    if (!read_file(base_dir + idx_file, h_idx)) return 1;
     if (h_ptr.empty()) {
-        std::cerr << graph << ".new_indptr is empty" << std::endl;
+        std::cerr << ptr_file << " is empty" << std::endl;
         return 1;
     }
     const int v_num = (int)h_ptr.size() - 1, e_num = (int)h_idx.size();
@@ -184,6 +194,7 @@ int main(int argc, char *argv[])
         if (a == "--graphs" && i + 1 < argc) base_dir = argv[++i];
         else if (a == "--meta" && i + 1 < argc) meta_dir = argv[++i];
         else if (a == "--save-state") save_state = true;
+        else if (a == "--natural") natural_order = true;
         else pos.push_back(a);
     }
     if (!base_dir.empty() && base_dir.back() != '/') base_dir += '/';

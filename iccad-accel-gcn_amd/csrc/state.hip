@@ -1,46 +1,42 @@
-// Saved preprocessing state: what accel_preprocess produced for one CSR, written to a
-// file and loaded into a new handle on the same CSR instead of being recomputed.
+// Saved preprocessing state: the part of accel_preprocess that a file can stand in for.
 //
-// Upstream persists its preprocessing the same way: block_level_partition.py:105-106
-// writes <graph>.block4 once and SPMM_ACCEL::do_test loads it on every call
-// (spmm_accel.cu:122).  Here the state is the block4 metadata plus the other products
-// of the GPU preprocessing: the degree-sort permutation, the sorted indptr, the launch
-// plan and the partial-sum slots of the split rows.  The sorted copy of the non-zeros is
-// not stored (it is as large as the CSR itself); it is gathered again from the caller's
-// arrays by two kernels.
+// Upstream persists its preprocessing as a file: block_level_partition.py:105-106 writes
+// <graph>.block4 once and SPMM_ACCEL::do_test loads it on every call (spmm_accel.cu:122).
+// Here every product of the preprocessing except one is rebuilt on the GPU faster than a
+// file of its size can be read (block4, the sorted indptr, the launch plan and the
+// partial-sum slots together take well under a millisecond for 125 M non-zeros), and the
+// sorted copy of the non-zeros is as large as the CSR itself.  The state therefore holds
+// the one product that is an input to all the others, the degree-sort permutation, plus
+// the plan options the handle was preprocessed with.  accel_load_state reads it and runs
+// the preprocessing with the sort replaced by the stored order.
 //
-// The file is keyed by content hashes of indptr and idx (computed on the GPU), so a
-// state saved for another graph is refused with ACCEL_ERR_META, and every stored array
-// carries its own hash, so a damaged file is refused before any kernel uses it.
-#include <cstring>
+// Nothing in the file is trusted: the stored order is accepted only if a kernel finds it
+// to be exactly the order the sort would produce for this CSR's indptr (that order is
+// unique), so a state of another matrix, of another library version or with flipped bits
+// is refused with ACCEL_ERR_META, and everything that indexes memory is computed afresh
+// by the code that is running.
 #include <chrono>
 #include <cstdio>
-#include <memory>
-#include <new>
-#include <vector>
+#include <cstring>
+#include <string>
 
 #include "internal.h"
 
 namespace accel {
 namespace {
 
-constexpr char kMagic[8] = {'A', 'C', 'G', 'C', 'N', 'S', 'T', '1'};
-constexpr uint32_t kStateVersion = 1;
-constexpr uint64_t kSeedIndptr = 0x11, kSeedIdx = 0x22, kSeedArray = 0x100;
-
-enum ArrayId { kPerm = 0, kSortedIndptr, kBlock4, kWork, kLongSlot, kNumArrays };
+constexpr char kMagic[8] = {'A', 'C', 'G', 'C', 'N', 'S', 'T', '2'};
+constexpr uint32_t kStateVersion = 2;
 
 struct StateHeader {
     char magic[8];
     uint32_t version, header_bytes;
+    int32_t library_version;          // accel_version() of the writer (informative)
+    int32_t identity_perm;            // 1: the rows were already in degree order, no permutation follows
     int64_t rows, cols, nnz;
-    uint64_t hash_indptr, hash_idx;
-    int64_t n_blocks, n_long_blocks, n_long_rows, n_zero_rows, n_units, n_long_units, n_split_rows,
-        n_big_rows, n_wide_rows;
-    int32_t max_degree, identity_perm, plan_unit, plan_split, plan_groups, plan_team, local,
-        waves_per_group;
-    int64_t words[kNumArrays];        // 4-byte words of each stored array (0: absent)
-    uint64_t hash[kNumArrays];        // content hash of each stored array
+    int32_t plan_unit_option, plan_split_option, plan_groups, plan_team_option, plan_queues_option;
+    int32_t reserved;
+    int64_t perm_words;               // rows, or 0 with identity_perm
     uint64_t header_hash;             // FNV-1a of this header with header_hash = 0
 };
 
@@ -58,59 +54,25 @@ struct File {
     ~File() { if (f) fclose(f); }
 };
 
-struct DevU64 {
-    uint64_t *p = nullptr;
-    ~DevU64() { if (p) (void)hipFree(p); }
-    int alloc(int n)
+struct PinnedBuf {   // host memory the GPU copies from and to directly
+    void *p = nullptr;
+    ~PinnedBuf() { if (p) (void)hipHostFree(p); }
+    int alloc(size_t bytes)
     {
-        if (hipMalloc(reinterpret_cast<void **>(&p), sizeof(uint64_t) * (size_t)n) != hipSuccess) {
+        if (hipHostMalloc(&p, bytes ? bytes : 4, hipHostMallocDefault) != hipSuccess) {
             (void)hipGetLastError();
             p = nullptr;
-            set_error("device allocation failed");
+            set_error("allocation of %zu bytes of pinned host memory failed", bytes);
             return ACCEL_ERR_ALLOC;
         }
         return ACCEL_OK;
     }
 };
 
-// hashes of several device arrays in one go: out_host[i] = hash of arrays[i]
-int hash_arrays(const void *const *arrays, const int64_t *words, const uint64_t *seeds, int n,
-                uint64_t *out_host)
-{
-    DevU64 d;
-    if (int rc = d.alloc(n)) return rc;
-    if (int rc = fill_u32(d.p, 0u, (size_t)n * 2, nullptr)) return rc;
-    for (int i = 0; i < n; i++)
-        if (int rc = hash_words_device(arrays[i], words[i], seeds[i], d.p + i, nullptr)) return rc;
-    ACCEL_HIP(hipMemcpy(out_host, d.p, sizeof(uint64_t) * (size_t)n, hipMemcpyDeviceToHost));
-    return ACCEL_OK;
-}
-
-int csr_hashes(const accel_handle *h, uint64_t *hash_indptr, uint64_t *hash_idx)
-{
-    const void *arrays[2] = {h->indptr, h->idx};
-    const int64_t words[2] = {h->rows + 1, h->nnz};
-    const uint64_t seeds[2] = {kSeedIndptr, kSeedIdx};
-    uint64_t out[2] = {0, 0};
-    if (int rc = hash_arrays(arrays, words, seeds, 2, out)) return rc;
-    *hash_indptr = out[0];
-    *hash_idx = out[1];
-    return ACCEL_OK;
-}
-
-void stored_arrays(const accel_handle *h, const void **arrays, int64_t *words)
-{
-    arrays[kPerm] = h->perm;
-    words[kPerm] = h->perm ? h->rows : 0;
-    arrays[kSortedIndptr] = h->s_indptr;
-    words[kSortedIndptr] = h->s_indptr ? h->rows + 1 : 0;
-    arrays[kBlock4] = h->block4;
-    words[kBlock4] = 4 * h->n_blocks;
-    arrays[kWork] = h->work;
-    words[kWork] = 4 * h->n_units;
-    arrays[kLongSlot] = h->long_slot;
-    words[kLongSlot] = h->long_slot ? h->n_split_rows + 1 : 0;
-}
+struct DevMem {
+    void *p = nullptr;
+    ~DevMem() { if (p) (void)hipFree(p); }
+};
 
 }  // namespace
 }  // namespace accel
@@ -129,23 +91,19 @@ int accel_save_state(const accel_handle *h, const char *path)
     std::memcpy(hd.magic, kMagic, sizeof kMagic);
     hd.version = kStateVersion;
     hd.header_bytes = (uint32_t)sizeof(StateHeader);
+    hd.library_version = accel_version();
+    hd.identity_perm = h->identity_perm ? 1 : 0;
     hd.rows = h->rows; hd.cols = h->cols; hd.nnz = h->nnz;
-    hd.n_blocks = h->n_blocks; hd.n_long_blocks = h->n_long_blocks; hd.n_long_rows = h->n_long_rows;
-    hd.n_zero_rows = h->n_zero_rows; hd.n_units = h->n_units; hd.n_long_units = h->n_long_units;
-    hd.n_split_rows = h->n_split_rows; hd.n_big_rows = h->n_big_rows; hd.n_wide_rows = h->n_wide_rows;
-    hd.max_degree = h->max_degree; hd.identity_perm = h->identity_perm ? 1 : 0;
-    hd.plan_unit = h->plan_unit; hd.plan_split = h->plan_split; hd.plan_groups = h->plan_groups;
-    hd.plan_team = h->plan_team ? 1 : 0; hd.local = h->local ? 1 : 0;
-    hd.waves_per_group = kWavesPerGroup;
-    const void *arrays[kNumArrays];
-    stored_arrays(h, arrays, hd.words);
-    if (h->rows > 0) {
-        if (int rc = csr_hashes(h, &hd.hash_indptr, &hd.hash_idx)) return rc;
-        uint64_t seeds[kNumArrays];
-        for (int i = 0; i < kNumArrays; i++) seeds[i] = kSeedArray + (uint64_t)i;
-        if (int rc = hash_arrays(arrays, hd.words, seeds, kNumArrays, hd.hash)) return rc;
-    }
+    hd.plan_unit_option = h->plan_unit_option; hd.plan_split_option = h->plan_split_option;
+    hd.plan_groups = h->plan_groups; hd.plan_team_option = h->plan_team_option;
+    hd.plan_queues_option = h->plan_queues_option;
+    hd.perm_words = h->identity_perm ? 0 : h->rows;
     hd.header_hash = header_hash(hd);
+    PinnedBuf host;
+    if (hd.perm_words > 0) {
+        if (int rc = host.alloc(sizeof(int32_t) * (size_t)hd.perm_words)) return rc;
+        ACCEL_HIP(hipMemcpy(host.p, h->perm, sizeof(int32_t) * (size_t)hd.perm_words, hipMemcpyDeviceToHost));
+    }
     // write to a temporary name and rename, so that a reader never sees half a file
     const std::string tmp = std::string(path) + ".tmp";
     {
@@ -153,36 +111,15 @@ int accel_save_state(const accel_handle *h, const char *path)
         out.f = fopen(tmp.c_str(), "wb");
         if (!out.f) { set_error("cannot create %s", tmp.c_str()); return ACCEL_ERR_IO; }
         bool ok = fwrite(&hd, sizeof hd, 1, out.f) == 1;
-        int rc = ACCEL_OK;
-        std::vector<uint32_t> host;
-        for (int i = 0; i < kNumArrays && ok && !rc; i++) {
-            if (hd.words[i] == 0) continue;
-            try {
-                host.resize((size_t)hd.words[i]);
-            } catch (const std::bad_alloc &) {
-                set_error("host allocation of %lld bytes failed", (long long)hd.words[i] * 4);
-                rc = ACCEL_ERR_ALLOC;
-                break;
-            }
-            const hipError_t e =
-                hipMemcpy(host.data(), arrays[i], sizeof(uint32_t) * host.size(), hipMemcpyDeviceToHost);
-            if (e != hipSuccess) {
-                set_error("download of the state failed: %s", hipGetErrorString(e));
-                rc = ACCEL_ERR_HIP;
-                break;
-            }
-            ok = fwrite(host.data(), sizeof(uint32_t), host.size(), out.f) == host.size();
-        }
+        if (ok && hd.perm_words > 0)
+            ok = fwrite(host.p, sizeof(int32_t), (size_t)hd.perm_words, out.f) == (size_t)hd.perm_words;
         ok = ok && fflush(out.f) == 0;
-        if (!rc && !ok) {
+        if (!ok) {
             set_error("write to %s failed", tmp.c_str());
-            rc = ACCEL_ERR_IO;
-        }
-        if (rc) {
             fclose(out.f);
             out.f = nullptr;
             (void)remove(tmp.c_str());
-            return rc;
+            return ACCEL_ERR_IO;
         }
     }
     if (rename(tmp.c_str(), path) != 0) {
@@ -204,7 +141,7 @@ int accel_load_state(accel_handle *h, const char *path)
     StateHeader hd;
     if (fread(&hd, sizeof hd, 1, in.f) != 1) { set_error("%s: truncated header", path); return ACCEL_ERR_IO; }
     if (std::memcmp(hd.magic, kMagic, sizeof kMagic) != 0 || hd.version != kStateVersion ||
-        hd.header_bytes != sizeof(StateHeader) || hd.waves_per_group != kWavesPerGroup) {
+        hd.header_bytes != sizeof(StateHeader)) {
         set_error("%s is not a state file of this library version", path);
         return ACCEL_ERR_META;
     }
@@ -218,24 +155,19 @@ int accel_load_state(accel_handle *h, const char *path)
                   (long long)h->cols, (long long)h->nnz);
         return ACCEL_ERR_META;
     }
-    // the header must be consistent with itself before anything is sized from it
-    const int64_t want[kNumArrays] = {hd.identity_perm ? 0 : hd.rows, hd.rows > 0 ? hd.rows + 1 : 0,
-                                      4 * hd.n_blocks, 4 * hd.n_units,
-                                      hd.rows > 0 ? hd.n_split_rows + 1 : 0};
-    bool sane = hd.n_blocks >= 0 && hd.n_units >= 0 && hd.n_split_rows >= 0 && hd.n_split_rows <= hd.rows &&
-                hd.n_big_rows >= 0 && hd.n_big_rows <= hd.n_split_rows && hd.n_wide_rows >= 0 &&
-                hd.n_wide_rows <= hd.rows && hd.n_zero_rows >= 0 &&
-                hd.n_zero_rows <= hd.rows && hd.n_long_units >= 0 && hd.n_long_units <= hd.n_units &&
-                hd.n_blocks <= hd.rows + hd.nnz && hd.n_units <= 0x7fffffffLL &&
-                hd.n_units % (kXcds * kWavesPerGroup) == 0 &&
-                (hd.plan_groups == 0 || hd.plan_groups == 8 || hd.plan_groups == 16 || hd.plan_groups == 32 ||
-                 hd.plan_groups == 64);
-    for (int i = 0; i < kNumArrays && sane; i++) sane = hd.words[i] == want[i];
+    // the header must be consistent with itself and hold options the setters would accept
+    auto unit_ok = [](int v) { return v == 0 || (v >= 16 && v <= kDegBound); };
+    const bool sane = (hd.identity_perm == 0 || hd.identity_perm == 1) &&
+                      hd.perm_words == (hd.identity_perm ? 0 : hd.rows) && unit_ok(hd.plan_unit_option) &&
+                      unit_ok(hd.plan_split_option) &&
+                      (hd.plan_groups == 0 || hd.plan_groups == 8 || hd.plan_groups == 16 ||
+                       hd.plan_groups == 32 || hd.plan_groups == 64) &&
+                      hd.plan_team_option >= 0 && hd.plan_team_option <= 2 &&
+                      (hd.plan_queues_option == 0 || hd.plan_queues_option == 1 || hd.plan_queues_option == kXcds);
     if (!sane) { set_error("%s: inconsistent header", path); return ACCEL_ERR_META; }
     // the file must be exactly as long as the header says, before anything is allocated from it
     {
-        int64_t expect = (int64_t)sizeof(StateHeader);
-        for (int i = 0; i < kNumArrays; i++) expect += 4 * hd.words[i];
+        const int64_t expect = (int64_t)sizeof(StateHeader) + 4 * hd.perm_words;
         const long at = ftell(in.f);
         if (at < 0 || fseek(in.f, 0, SEEK_END) != 0) { set_error("%s: cannot seek", path); return ACCEL_ERR_IO; }
         const long len = ftell(in.f);
@@ -246,91 +178,39 @@ int accel_load_state(accel_handle *h, const char *path)
             return ACCEL_ERR_IO;
         }
     }
-
-    release_products(h);
-    if (h->rows == 0) {
-        h->identity_perm = true;
-        h->ready = true;
-        return ACCEL_OK;
-    }
-    uint64_t hi = 0, hx = 0;
-    if (int rc = csr_hashes(h, &hi, &hx)) return rc;
-    if (hi != hd.hash_indptr || hx != hd.hash_idx) {
-        set_error("%s was saved for a different CSR (content hash of %s differs)", path,
-                  hi != hd.hash_indptr ? "indptr" : "idx");
-        return ACCEL_ERR_META;
-    }
-    // upload the stored arrays; on any failure the handle is left without products
-    void *dev[kNumArrays] = {};
-    auto fail = [&](int rc) {
-        for (auto p : dev)
-            if (p) (void)hipFree(p);
-        return rc;
-    };
-    std::vector<uint32_t> host;
-    for (int i = 0; i < kNumArrays; i++) {
-        if (hd.words[i] == 0) continue;
-        try {
-            host.resize((size_t)hd.words[i]);
-        } catch (const std::bad_alloc &) {
-            set_error("host allocation of %lld bytes failed", (long long)hd.words[i] * 4);
-            return fail(ACCEL_ERR_ALLOC);
-        }
-        if (fread(host.data(), sizeof(uint32_t), host.size(), in.f) != host.size()) {
-            set_error("%s: truncated", path);
-            return fail(ACCEL_ERR_IO);
-        }
-        if (hipMalloc(&dev[i], sizeof(uint32_t) * host.size()) != hipSuccess) {
+    // the file goes into pinned memory, from which the GPU copies it in one transfer
+    PinnedBuf host;
+    DevMem dev;
+    SavedOrder order{hd.identity_perm != 0, nullptr};
+    if (hd.perm_words > 0) {
+        const size_t bytes = sizeof(int32_t) * (size_t)hd.perm_words;
+        if (int rc = host.alloc(bytes)) return rc;
+        if (fread(host.p, 1, bytes, in.f) != bytes) { set_error("%s: truncated", path); return ACCEL_ERR_IO; }
+        if (hipMalloc(&dev.p, bytes) != hipSuccess) {
             (void)hipGetLastError();
-            dev[i] = nullptr;
-            set_error("device allocation of %zu bytes failed", sizeof(uint32_t) * host.size());
-            return fail(ACCEL_ERR_ALLOC);
+            dev.p = nullptr;
+            set_error("device allocation of %zu bytes failed", bytes);
+            return ACCEL_ERR_ALLOC;
         }
-        if (hipMemcpy(dev[i], host.data(), sizeof(uint32_t) * host.size(), hipMemcpyHostToDevice) != hipSuccess) {
-            set_error("upload of the saved state failed");
-            return fail(ACCEL_ERR_HIP);
-        }
+        ACCEL_HIP(hipMemcpyAsync(dev.p, host.p, bytes, hipMemcpyHostToDevice, nullptr));
+        order.perm_dev = static_cast<const uint32_t *>(dev.p);
     }
-    {
-        uint64_t seeds[kNumArrays], got[kNumArrays];
-        for (int i = 0; i < kNumArrays; i++) seeds[i] = kSeedArray + (uint64_t)i;
-        if (int rc = hash_arrays(dev, hd.words, seeds, kNumArrays, got)) return fail(rc);
-        for (int i = 0; i < kNumArrays; i++)
-            if (got[i] != hd.hash[i]) {
-                set_error("%s: stored array %d does not match its hash (damaged file)", path, i);
-                return fail(ACCEL_ERR_META);
-            }
-    }
-    h->perm = static_cast<int32_t *>(dev[kPerm]);
-    h->s_indptr = static_cast<int32_t *>(dev[kSortedIndptr]);
-    h->block4 = static_cast<int32_t *>(dev[kBlock4]);
-    h->work = static_cast<int32_t *>(dev[kWork]);
-    h->long_slot = static_cast<int32_t *>(dev[kLongSlot]);
-    h->identity_perm = hd.identity_perm != 0;
-    h->n_blocks = hd.n_blocks; h->n_long_blocks = hd.n_long_blocks; h->n_long_rows = hd.n_long_rows;
-    h->n_zero_rows = hd.n_zero_rows; h->n_units = hd.n_units; h->n_long_units = hd.n_long_units;
-    h->n_split_rows = hd.n_split_rows; h->n_big_rows = hd.n_big_rows; h->n_wide_rows = hd.n_wide_rows;
-    h->max_degree = hd.max_degree;
-    h->plan_unit = hd.plan_unit; h->plan_split = hd.plan_split; h->plan_groups = hd.plan_groups;
-    h->plan_team = hd.plan_team != 0; h->local = hd.local != 0;
-    // non-zeros of the rows that are not split = sorted indptr at the first split row
-    const int64_t first_long = h->rows - h->n_split_rows;
-    int32_t nz_short32 = 0;
-    int rc = ACCEL_OK;
-    if (hipMemcpy(&nz_short32, h->s_indptr + first_long, sizeof(int32_t), hipMemcpyDeviceToHost) != hipSuccess) {
-        set_error("read-back of the sorted indptr failed");
-        rc = ACCEL_ERR_HIP;
-    }
-    if (!rc && (nz_short32 < 0 || (int64_t)nz_short32 > h->nnz)) {
-        set_error("%s: sorted indptr out of range", path);
-        rc = ACCEL_ERR_META;
-    }
-    if (!rc) rc = rebuild_sorted_csr(h, nz_short32, nullptr);
+    release_products(h);
+    // the options of the state replace the handle's, so that the handle ends up as the one
+    // that was saved; they come back if the load fails
+    const int keep[5] = {h->plan_unit_option, h->plan_split_option, h->plan_groups, h->plan_team_option,
+                         h->plan_queues_option};
+    h->plan_unit_option = hd.plan_unit_option; h->plan_split_option = hd.plan_split_option;
+    h->plan_groups = hd.plan_groups; h->plan_team_option = hd.plan_team_option;
+    h->plan_queues_option = hd.plan_queues_option;
+    const int rc = preprocess_device(h, &order);
+    (void)hipStreamSynchronize(nullptr);            // the staging buffers go away with this scope
     if (rc) {
         release_products(h);
+        h->plan_unit_option = keep[0]; h->plan_split_option = keep[1]; h->plan_groups = keep[2];
+        h->plan_team_option = keep[3]; h->plan_queues_option = keep[4];
         return rc;
     }
-    h->ready = true;
     h->preprocess_ms =
         std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     return ACCEL_OK;

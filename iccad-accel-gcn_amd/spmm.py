@@ -60,13 +60,17 @@ class AccelSpMM:
 
     # -- preprocess ---------------------------------------------------------
     def preprocess(self, plan_unit: int | None = None, plan_groups: int | None = None,
-                   plan_split: int | None = None, plan_team: int | None = None) -> "AccelSpMM":
+                   plan_split: int | None = None, plan_team: int | None = None,
+                   plan_queues: int | None = None) -> "AccelSpMM":
         """Degree sort, block4 metadata and launch plan on the GPU.  ``plan_unit``
         (16..384) overrides the automatic choice of non-zeros per unit,
         ``plan_groups`` (8, 16, 32, 64) that of column groups for split rows,
         ``plan_split`` (16..384) the row length above which rows are split,
         ``plan_team`` (1: one wavefront per unit, 2: one workgroup per unit) who
-        works on a unit."""
+        works on a unit, ``plan_queues`` (8 or 1) the number of interleaved queues of
+        the plan (default: from the shape of the device)."""
+        if plan_queues is not None:
+            check(lib().accel_set_plan_queues(self._h, int(plan_queues)))
         if plan_team is not None:
             check(lib().accel_set_plan_team(self._h, int(plan_team)))
         if plan_unit is not None:
@@ -82,13 +86,14 @@ class AccelSpMM:
         return self
 
     def save_state(self, path) -> None:
-        """Write what preprocess() built (block4, permutation, launch plan) to ``path``."""
+        """Write the degree-sort order and the plan options of this operator to ``path``."""
         self.info
         check(lib().accel_save_state(self._h, str(path).encode()))
 
     def load_state(self, path) -> "AccelSpMM":
-        """Take the place of preprocess(): load a state saved for the same CSR.
-        Raises AccelError (ERR_META) if the file belongs to another CSR or is damaged."""
+        """Take the place of preprocess(): the preprocessing with the sort replaced by the
+        order saved for the same CSR.  Raises AccelError (ERR_META) if the file belongs to
+        another CSR or is damaged."""
         check(lib().accel_load_state(self._h, str(path).encode()))
         info = Info()
         check(lib().accel_get_info(self._h, C.byref(info)))
@@ -110,6 +115,15 @@ class AccelSpMM:
             check(lib().accel_update_values(self._h, _lib.dev_ptr(values, self.nnz * 4, "values"), _lib.PTR_DEVICE))
             if self._keep is not None and len(self._keep) == 3:
                 self._keep = (self._keep[0], self._keep[1], values)
+        return self
+
+    def update_values_async(self, values, stream=None) -> "AccelSpMM":
+        """New values for the same structure from a device array, queued on ``stream``
+        without waiting (see accel_update_values_async)."""
+        self.info
+        check(lib().accel_update_values_async(self._h, _lib.dev_ptr(values, self.nnz * 4, "values"), ptr(stream)))
+        if self._keep is not None and len(self._keep) == 3:
+            self._keep = (self._keep[0], self._keep[1], values)
         return self
 
     def set_panel(self, columns: int) -> None:
@@ -272,7 +286,10 @@ class SpmmAccel:
         self.val, self.vin, self.vout = val, vin, vout
         self.num_v, self.num_e, self.dim = int(num_v), int(num_e), int(dim)
         self.meta_dir = Path(meta_dir)
-        self.save_state = False        # True: write <meta_dir>/<graph>.accelstate after preprocessing
+        # True: use <meta_dir>/<graph>.accelstate: load it instead of sorting when it belongs
+        # to this CSR, write it after preprocessing otherwise.  Off by default: on this GPU
+        # the load is not faster than the preprocessing.
+        self.save_state = False
         self.state_loaded = False
         self._op = AccelSpMM(ptr_, idx, val, self.num_v, device=True, n_rows=self.num_v, nnz=self.num_e)
         self._ready = False
@@ -280,15 +297,15 @@ class SpmmAccel:
     def _preprocess(self):
         if self._ready:
             # upstream's kernel reads val on every launch (spmm_accel.cu:75): a caller may have
-            # rewritten the array since the last call
-            self._op.update_values(self.val)
+            # rewritten the array since the last call; one kernel on the stream of the runs
+            self._op.update_values_async(self.val)
             return
         # the saved state of an earlier run takes the place of the preprocessing, as
         # upstream's operator loads its metadata file (spmm_accel.cu:122); a state that
         # does not belong to this CSR is a stale cache entry, not an error
         state = self.meta_dir / f"{self._graph}.accelstate"
         loaded = False
-        if state.exists():
+        if self.save_state and state.exists():
             try:
                 self._op.load_state(state)
                 loaded = True

@@ -296,11 +296,13 @@ def workload(spec):
 
 
 def export_upstream_layout(spec_or_graph, graphs_dir, name=None):
-    """Write a workload the way upstream's programs read their datasets (main.cu:62-63,
+    """Write a workload the way upstream's programs read their datasets (main.cu:62-65,
     block_level_partition.py:26-32): ``<name>.config`` (presence only), ``<name>.new_indptr``
     and ``<name>.new_indices`` as raw little-endian int32, rows in ascending degree order
-    (ties keep their order).  Values are not part of the layout (upstream fills ones,
-    main.cu:114).  The adjacency must be square.  Returns the stem written."""
+    (ties keep their order), and ``<name>.graph.ptrdump`` / ``<name>.graph.edgedump``, the
+    same matrix with its rows in the workload's own order (column ids are the same in both
+    pairs).  Values are not part of the layout (upstream fills ones, main.cu:114).  The
+    adjacency must be square.  Returns the stem written."""
     from pathlib import Path
     g = workload(spec_or_graph) if isinstance(spec_or_graph, str) else spec_or_graph
     if g.n_rows != g.n_cols:
@@ -318,6 +320,8 @@ def export_upstream_layout(spec_or_graph, graphs_dir, name=None):
     (out / f"{name}.config").write_text("")
     sip.astype("<i4").tofile(out / f"{name}.new_indptr")
     g.indices[src].astype("<i4").tofile(out / f"{name}.new_indices")
+    np.asarray(g.indptr).astype("<i4").tofile(out / f"{name}.graph.ptrdump")
+    np.asarray(g.indices).astype("<i4").tofile(out / f"{name}.graph.edgedump")
     return name
 
 

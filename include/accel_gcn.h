@@ -135,17 +135,21 @@ int accel_set_plan_team(accel_handle *h, int mode);
 
 /* Saved preprocessing state.  Upstream persists its preprocessing as a file
  * (block_level_partition.py:105-106 writes <graph>.block4) and its operator loads
- * that file instead of recomputing (spmm_accel.cu:122).  accel_save_state writes
- * what accel_preprocess built for this handle: the block4 metadata, the degree-sort
- * permutation, the sorted indptr, the launch plan and the partial-sum slots (not the
- * sorted copy of the non-zeros, which is regathered on load).  accel_load_state takes
- * the place of accel_preprocess on a handle created on the same CSR: the file is
- * keyed by content hashes of indptr and idx, computed on the GPU; a file saved for
- * another CSR, by another library version, or damaged (every stored array carries
- * a hash) gives ACCEL_ERR_META and leaves the handle un-preprocessed, a missing or
- * short file ACCEL_ERR_IO.  After a successful load the handle behaves exactly as
- * after accel_preprocess with the options the state was saved with (the results of
- * accel_run are the same bits); accel_info.preprocess_ms is the time of the load. */
+ * that file instead of recomputing (spmm_accel.cu:122).  On this GPU every product of
+ * accel_preprocess but one is rebuilt faster than a file of its size can be read, so
+ * accel_save_state writes that one, the degree-sort permutation (4 bytes per row), and
+ * the plan options of the handle.  accel_load_state takes the place of accel_preprocess
+ * on a handle created on the same CSR: it runs the preprocessing with the sort replaced
+ * by the stored order.  Nothing in the file is trusted: the order is used only after a
+ * kernel has found it to be exactly the degree order of this CSR (ascending degree,
+ * ties by row id: there is only one), so a file saved for another matrix, written by
+ * another library version or damaged gives ACCEL_ERR_META and leaves the handle
+ * un-preprocessed and its options as they were; a missing or short file gives
+ * ACCEL_ERR_IO.  After a successful load the handle is the one that was saved: the same
+ * options, and the results of accel_run are the same bits; accel_info.preprocess_ms is
+ * the time of the load.  The load is not faster than accel_preprocess (reading the file
+ * costs more than the sort it replaces); it exists for callers that want the operator's
+ * state to travel with the graph, as upstream's metadata file does. */
 int accel_save_state(const accel_handle *h, const char *path);
 int accel_load_state(accel_handle *h, const char *path);
 
@@ -153,19 +157,43 @@ int accel_load_state(accel_handle *h, const char *path);
  * at accel_create), e.g. edge weights that change between training steps.  Upstream's
  * kernel reads the caller's `val` on every launch (spmm_accel.cu:75), so a caller that
  * rewrites the array sees the new weights at once; this library computes from its
- * degree-sorted copy, which this call refreshes (one gather pass over the non-zeros,
- * about half the time of accel_preprocess; sort, metadata and launch plan are kept).
- * val: nnz floats in the order of the CSR given to accel_create; flags says where it
- * lives (ACCEL_PTR_HOST or ACCEL_PTR_DEVICE).  A handle that uploaded its CSR copies
- * the values into its own array; a handle that borrows device arrays needs a device
- * array and borrows that one from now on (it may be the same array, rewritten in
- * place).  Synchronous, and it waits for all work on the device first: do not call it
- * while a stream is capturing.  A saved state holds no values and stays valid.  The
- * sorted copy is rewritten where it is, so HIP graphs captured from runs of this handle
- * stay valid and compute with the new values (exception: a CSR that was already sorted
- * and has no split row is read in place, so passing a different array changes the
- * address a captured run reads). */
+ * degree-sorted copy, which these calls bring up to date: one kernel that gathers the
+ * values through a map from sorted position to the caller's position (sort, metadata
+ * and launch plan are kept).  The first update of a handle builds that map (one device
+ * allocation of 4 bytes per non-zero, kept until the next accel_preprocess); later ones
+ * allocate nothing.
+ *
+ * accel_update_values_async: val_dev = nnz floats on the device in the order of the CSR
+ * given to accel_create; the kernel is queued on `stream` (a hipStream_t, NULL = default
+ * stream) and the call returns without waiting.  The handle orders it on the device
+ * behind its own runs that are still in flight on other streams, and later runs on other
+ * streams behind it, so "update, then run" needs no host synchronisation whatever the
+ * streams are.  It can be captured into a HIP graph together with the runs that follow
+ * (after one update outside the capture has built the map; a capturing stream is only
+ * ordered against itself).  A handle that uploaded its CSR also copies the values into
+ * its own array (same stream); a handle that borrows device arrays borrows val_dev from
+ * now on (it may be the same array, rewritten in place).
+ *
+ * accel_update_values: the same for an array in host memory (ACCEL_PTR_HOST: copied to the
+ * device first; only for handles that own their CSR) or on the device (ACCEL_PTR_DEVICE),
+ * on the default stream, and it returns when the update is done.  Not while capturing.
+ *
+ * A saved state holds no values and stays valid.  The sorted copy is rewritten where it
+ * is, so HIP graphs captured from runs of this handle stay valid and compute with the new
+ * values (exception: a CSR that was already sorted and has no split row is read in place,
+ * so passing a different array changes the address a captured run reads). */
 int accel_update_values(accel_handle *h, const float *val, int flags);
+int accel_update_values_async(accel_handle *h, const float *val_dev, void *stream);
+
+/* Interleaved queues of the launch plan (no counterpart upstream, whose grid is the block4
+ * list in order, spmm_accel.cu:128).  The plan is laid out for the way the whole MI355X
+ * hands out workgroups: workgroup i runs on die i % 8, so the list is eight interleaved
+ * queues, one per die and its L2 (see accel_get_plan).  0 (the default) = from the device
+ * the handle was created on: 8 when it has the 256 compute units of the whole GPU, 1 on
+ * any other shape (a partition of the GPU, where that mapping does not hold): the same
+ * units in one queue, column group after column group.  1 or 8 force the layout.  Call
+ * before accel_preprocess; accel_info.plan_queues tells what was used. */
+int accel_set_plan_queues(accel_handle *h, int queues);
 
 /* Column panels (no counterpart upstream, which always walks all N columns of a row
  * at once, spmm_accel.cu:37-48): one accel_run computes Y one panel of `columns`
@@ -195,6 +223,7 @@ typedef struct accel_info {
     int32_t plan_groups;    /* 0: column groups chosen per row from its length; 8..64: forced */
     int32_t plan_split_nz;  /* rows with more non-zeros than this are cut into pieces */
     int32_t plan_team;      /* 1: a unit is worked on by a whole workgroup, 0: by one wavefront */
+    int32_t plan_queues;    /* interleaved queues of the launch plan: 8 (one per die) or 1 */
 } accel_info;
 int accel_get_info(const accel_handle *h, accel_info *out);
 
@@ -210,7 +239,8 @@ int accel_get_sorted_csr(const accel_handle *h, int32_t *indptr, int32_t *idx, f
  * accel_info.plan_team is 1; the list has the same form).  x <= 384: a block4 entry of
  * whole rows, verbatim.  x > 384: a piece of a long row: partial-sum slot
  * x - 385, sorted row y, first non-zero z, length w <= 384.  w == 0: padding.
- * Workgroup i runs on die i % 8, so units 4*i .. 4*i+3 belong to queue i % 8;
+ * With accel_info.plan_queues == 1 the list is one queue in the order described below;
+ * with 8: workgroup i runs on die i % 8, so units 4*i .. 4*i+3 belong to queue i % 8;
  * the pieces of split rows in queue g only hold columns c with (c >> 3) & 7 == g,
  * ordered by column group ((c >> 3) & (groups - 1)) when there are more than 8, and
  * inside a group by the caller's row id (rows of 8 groups; longer rows: largest
@@ -230,10 +260,15 @@ int accel_get_plan(const accel_handle *h, int32_t *out, int64_t cap_units, int64
  * are in the caller's original row order.  Asynchronous on `stream` (a
  * hipStream_t, NULL = default stream); X and Y are device pointers: an address the
  * GPU cannot read, or an allocation too small for cols x N (X) or rows x N (Y) floats,
- * is refused with ACCEL_ERR_ARG where the runtime can tell.  One handle runs on one
- * stream at a time: its partial-sum buffer is shared, and a run on a second stream
- * while the previous one is still in flight returns ACCEL_ERR_STATE (runs queued on
- * the same stream are ordered and fine; distinct handles are independent). */
+ * is refused with ACCEL_ERR_ARG where the runtime can tell (it is asked on every call,
+ * except while `stream` is capturing: the runtime answers no such query during a capture),
+ * and a call with another GPU current than the one the handle was created on with
+ * ACCEL_ERR_STATE.  The partial-sum buffer of a matrix with split rows is shared by all
+ * runs of the handle: a run on another stream than the previous one is made to wait, on
+ * the device, for what that stream held at the time of the call (no error, no host
+ * wait; runs on one stream are ordered anyway; distinct handles are independent).  A
+ * stream that is capturing is not ordered against other streams: the caller orders a
+ * graph against other uses of the handle. */
 int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream);
 
 /* run with the rest of a GCN layer fused into the store: Y = act(A X + bias).
@@ -299,9 +334,11 @@ int accel_reserve(accel_handle *h, int32_t max_N);
 int accel_run_static(accel_handle *h, const float *X, float *Y, int32_t N, void *stream);
 
 /* Timing protocol of SPMM_BASE::timing_body (spmm_base.h:34-63) with HIP
- * events on `stream`: `warmup` untimed runs, then `iters` runs each bracketed
- * by events.  ms_total[i] covers everything accel_run launches; ms_main[i]
- * (optional) only the gather kernel.  Either array may be NULL. */
+ * events on `stream`: `warmup` untimed runs, then `iters` runs queued back to back,
+ * each bracketed by two recorded events.  ms_total[i] covers everything accel_run
+ * launches; ms_main[i] (optional) only the gather kernel, taken from events bound to
+ * that kernel's own start and end (hipExtLaunchKernel), which put nothing between the
+ * kernels of a run.  Either array may be NULL. */
 int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup, int iters,
                float *ms_total, float *ms_main, void *stream);
 

@@ -40,10 +40,11 @@ public:
     /* Directory searched for "<graph>.block4" (default: upstream's relative path). */
     void set_meta_dir(const std::string &dir) { meta_dir = dir; }
     /* Preprocessing cache, the counterpart of upstream loading its metadata file on every
-     * do_test (spmm_accel.cu:122): "<meta_dir><graph>.accelstate", written by
-     * accel_save_state, is loaded instead of preprocessing when it belongs to this CSR
-     * (keyed by content hashes); otherwise the preprocessing runs and, after
-     * set_save_state(true), writes that file.  loaded_from_state() tells which happened. */
+     * do_test (spmm_accel.cu:122).  Off by default (on this GPU the preprocessing is as fast as
+     * reading a file).  After set_save_state(true): "<meta_dir><graph>.accelstate", written by
+     * accel_save_state, is used instead of sorting when it belongs to this CSR (the stored
+     * order is checked on the GPU); otherwise the preprocessing runs and writes that file.
+     * loaded_from_state() tells which happened. */
     void set_save_state(bool on) { save_state = on; }
     bool loaded_from_state() const { return from_state; }
     /* Text of the last error ("" if none). */

@@ -15,7 +15,8 @@ EXE = ROOT / "iccad-accel-gcn_amd" / "bin" / "spmm_test"
 
 def write_graph(tmp, name, seed, n_long=3):
     """<name>.config/.new_indptr/.new_indices in upstream's layout (degree-sorted
-    rows, raw int32), plus the matching <name>.block4."""
+    rows, raw int32), the same matrix in its own row order as <name>.graph.ptrdump /
+    .graph.edgedump (main.cu:64-65), plus the matching <name>.block4."""
     g0 = helpers.graph_from_degrees(helpers.degree_mix(seed=seed, n_long=n_long), seed=seed)
     n = g0.n_rows
     # square adjacency, as upstream assumes (vin has v_num rows)
@@ -28,6 +29,8 @@ def write_graph(tmp, name, seed, n_long=3):
     (graphs / f"{name}.config").write_text("")
     sip.astype("<i4").tofile(graphs / f"{name}.new_indptr")
     six.astype("<i4").tofile(graphs / f"{name}.new_indices")
+    g0.indptr.astype("<i4").tofile(graphs / f"{name}.graph.ptrdump")
+    g0.indices.astype("<i4").tofile(graphs / f"{name}.graph.edgedump")
     po.partition_closed_form(sip).astype("<i4").tofile(meta / f"{name}.block4")
     return graphs, meta
 
@@ -106,3 +109,30 @@ def test_cli_saved_state_is_loaded_by_the_next_run(gpu, tmp_path):
                            capture_output=True, text=True, timeout=120)
     assert third.returncode == 0, third.stdout + third.stderr
     assert "loaded from saved state" not in third.stderr and "validation pass!" in third.stdout
+
+
+@pytest.mark.gpu
+def test_cli_natural_order_input(gpu, tmp_path):
+    """--natural reads <g>.graph.ptrdump / .graph.edgedump (main.cu:64-65) and gives that CSR
+    to the operator, which sorts it itself: the same validation passes through both inputs,
+    and the .block4 file written for the sorted rows still describes the partition."""
+    graphs, meta = write_graph(tmp_path, "mix", seed=15)
+    base = [str(EXE), "--graphs", str(graphs), "--meta", str(meta)]
+    for extra in ([], ["--natural"]):
+        r = subprocess.run(base + extra + ["mix", "40"], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, r.stdout + r.stderr
+        assert "validation pass!" in r.stdout and re.search(r"^0/0 mix 40 accel ", r.stdout, re.M)
+    # unsorted input has a real permutation to save: the next run takes the order from the file
+    cmd = base + ["--natural", "--save-state", "mix", "40"]
+    first = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+    assert first.returncode == 0 and "loaded from saved state" not in first.stderr
+    assert (meta / "mix.accelstate").stat().st_size > 4 * (np.fromfile(graphs / "mix.graph.ptrdump", "<i4").size - 1)
+    second = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+    assert second.returncode == 0, second.stdout + second.stderr
+    assert "loaded from saved state" in second.stderr and "validation pass!" in second.stdout
+    # the state of the natural order does not fit the pre-sorted files: ignored, recomputed
+    third = subprocess.run(base + ["--save-state", "mix", "40"], capture_output=True, text=True, timeout=120)
+    assert third.returncode == 0, third.stdout + third.stderr
+    assert "loaded from saved state" not in third.stderr and "validation pass!" in third.stdout
+    missing = subprocess.run(base + ["--natural", "nosuch", "40"], capture_output=True, text=True, timeout=120)
+    assert missing.returncode != 0

@@ -189,14 +189,16 @@ def check_plan(op, n_cols):
     """The launch plan covers every non-zero exactly once; units of whole rows stay
     inside one block4 entry and hold at most plan_unit non-zeros (or one row); pieces of
     split rows hold at most plan_unit non-zeros (the split threshold, if that is larger)
-    of one column group and are queued on the die that owns that group."""
-    unit, split = op.info.plan_unit_nz, op.info.plan_split_nz
+    of one column group and are queued on the die that owns that group.  With one queue
+    (plan_queues == 1) the same order holds for the list as a whole."""
+    unit, split, nq = op.info.plan_unit_nz, op.info.plan_split_nz, op.info.plan_queues
+    assert nq in (1, 8)
     piece = max(unit, split)
     plan = op.plan().astype(np.int64)
     b4 = op.block4().astype(np.int64)
     sip, six, _ = op.sorted_csr()
     deg = np.diff(sip)
-    assert plan.shape[0] % 32 == 0 and plan.shape[0] == op.info.n_plan_units      # 8 queues x 4 wavefronts
+    assert plan.shape[0] % (4 * nq) == 0 and plan.shape[0] == op.info.n_plan_units   # queues x 4 wavefronts
     live = plan[plan[:, 3] != 0]
     short = live[live[:, 0] <= 384]
     long_ = live[live[:, 0] > 384]
@@ -218,8 +220,8 @@ def check_plan(op, n_cols):
     if unit == 384:
         assert sorted(map(tuple, short)) == sorted(map(tuple, b4[b4[:, 0] <= split]))   # entries verbatim
     assert np.all(covered == 1)
-    # queue of unit e is (e // 4) % 8
-    queue = (np.arange(plan.shape[0]) // 4) % 8
+    # queue of unit e is (e // 4) % 8 (one queue: 0)
+    queue = (np.arange(plan.shape[0]) // 4) % nq
     # the plan orders by the caller's row id in bands: the id's top 16 bits
     shift = 0
     while (max(deg.size, 1) - 1) >> shift >= 65536:
@@ -230,7 +232,7 @@ def check_plan(op, n_cols):
         x, y, z, w = plan[e]
         groups = po.row_groups(int(deg[y]), op.info.plan_groups)
         fine = po.column_group(six[z:z + w], groups)
-        assert np.all(fine == fine[0]) and fine[0] % 8 == queue[e]   # one group, on its die
+        assert np.all(fine == fine[0]) and fine[0] % nq == queue[e]  # one group, on its die
         # a die takes the rows with the most groups first and its groups in turn; inside a group
         # the rows follow the caller's row ids (8-group rows) or come largest first (longer rows)
         key = (-groups, int(fine[0]),
@@ -250,7 +252,7 @@ def check_plan(op, n_cols):
     perm = op.perm()
     light_nz = max(24, unit // 4)
     keys = []
-    for q in range(8):
+    for q in range(nq):
         mine = plan[queue == q]
         mine = mine[mine[:, 3] != 0]
         is_short = mine[:, 0] <= 384
@@ -268,18 +270,18 @@ def check_plan(op, n_cols):
         if n_tail and light[:in_line].any():             # held back: the light units with the highest ids
             assert k[in_line:].min() >= k[:in_line][light[:in_line]].max()
         keys.append(k)
-    for q in range(7):                                  # queue q's rows all precede queue q + 1's
+    for q in range(nq - 1):                             # queue q's rows all precede queue q + 1's
         later = np.concatenate(keys[q + 1:])
         if keys[q].size and later.size:
             assert keys[q].max() <= later.min()
     # ... and the shares level the load: cost = non-zeros + rows + 8 per unit, + 8 per piece
-    load = np.zeros(8)
+    load = np.zeros(nq)
     for e in np.flatnonzero(plan[:, 3] != 0):
         x, y, z, w = plan[e]
         load[queue[e]] += (w + 9) if x > 384 else (x + 1) * (w & 0xFFFF) + 8
     heaviest_unit = 384 + 64 + 8
     short_load = np.array([sum((d + 1) * (i & 0xFFFF) + 8 for d, r, l, i in plan[queue == q] if 0 < d <= 384 and i)
-                           for q in range(8)])
+                           for q in range(nq)])
     with_short = short_load > 0
     if with_short.sum() > 1:
         # queues that received whole-row units end up within a few units of each other
@@ -294,8 +296,35 @@ def test_launch_plan(gpu, seed, n_long, team):
     g = helpers.graph_from_degrees(helpers.degree_mix(seed=seed, n_long=n_long), seed=seed)
     op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_team=team)
     assert (op.info.plan_unit_nz, op.info.plan_split_nz) == ((48, 384) if team == 2 else (48, 48))
+    assert op.info.plan_queues == 8                      # the whole GPU: one queue per die
     check_plan(op, g.n_cols)
     op.close()
+
+
+@pytest.mark.parametrize("team", [1, 2])
+@pytest.mark.parametrize("seed,n_long", [(3, 0), (4, 9)])
+def test_launch_plan_in_one_queue(gpu, seed, n_long, team):
+    """The layout for a device that is not the whole GPU (a partition, where "workgroup i
+    runs on die i % 8" does not hold), forced here: the same units in plain order, column
+    group after column group, and the same product."""
+    from oracle import spmm_oracle as so
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=seed, n_long=n_long, zeros=5), seed=seed)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_team=team, plan_queues=1)
+    assert op.info.plan_queues == 1
+    check_plan(op, g.n_cols)
+    ref = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_team=team)
+    assert np.array_equal(op.block4(), ref.block4()) and np.array_equal(op.perm(), ref.perm())
+    assert sorted(map(tuple, op.plan()[op.plan()[:, 3] != 0])) == sorted(map(tuple, ref.plan()[ref.plan()[:, 3] != 0]))
+    for N in (16, 64, 100):
+        X = np.random.default_rng(N).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+        Y = op.matmul(X)
+        assert so.check(Y, g.indptr, g.indices, g.values, X) <= so.TOL
+        assert np.array_equal(Y.view(np.uint32), ref.matmul(X).view(np.uint32))   # same units, same sums
+    with pytest.raises(gpu.AccelError) as e:
+        gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_queues=4)
+    assert e.value.status == gpu._lib.ERR_ARG
+    op.close()
+    ref.close()
 
 
 def test_launch_plan_row_bands(gpu):

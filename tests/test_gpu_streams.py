@@ -151,36 +151,161 @@ def test_captured_graph_sees_updated_values(gpu, hip):
     dX.close(); dY.close(); op.close()
 
 
-def test_second_stream_is_refused_while_the_first_run_is_in_flight(gpu, hip):
+def test_second_stream_waits_for_the_first_on_the_device(gpu, hip):
     """The partial-sum buffer of a handle is shared by its runs: a run on another stream
-    while the previous one has not finished is an error, not silent corruption."""
+    than the previous one is ordered behind it on the device (no error, no host wait), so
+    runs queued on two streams give what they give one after the other."""
     g = gpu.synthetic.cfg2()
     N = 128
     X = gpu.synthetic.dense_operand("cfg2", g.n_cols, N)
+    X2 = np.ascontiguousarray(-2.0 * X)
     op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
     assert op.info.n_split_rows > 0
-    dX, dY = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer(g.n_rows * N * 4)
+    dX, dX2 = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer.from_numpy(X2)
+    dY, dY2 = gpu.DeviceBuffer(g.n_rows * N * 4), gpu.DeviceBuffer(g.n_rows * N * 4)
+    op.run(dX, dY, N)
+    op.run(dX2, dY2, N)
+    op.synchronize()
+    want, want2 = dY.to_numpy(np.float32, (g.n_rows, N)), dY2.to_numpy(np.float32, (g.n_rows, N))
+    assert so.check(want, g.indptr, g.indices, g.values, X) <= so.TOL
     s1, s2 = C.c_void_p(), C.c_void_p()
     ok(hip.hipStreamCreate(C.byref(s1)))
     ok(hip.hipStreamCreate(C.byref(s2)))
+    for rep in range(3):
+        dY.fill_u32(0x7FC00000)
+        dY2.fill_u32(0x7FC00000)
+        op.synchronize()
+        for _ in range(100):                              # some 15 ms of queued work on s1
+            op.run(dX, dY, N, stream=s1.value)
+        op.run(dX2, dY2, N, stream=s2.value)              # queued at once; waits on the device
+        for _ in range(20):                               # and back and forth, never waiting on the host
+            op.run(dX, dY, N, stream=s1.value)
+            op.run(dX2, dY2, N, stream=s2.value)
+        ok(hip.hipStreamSynchronize(s1))
+        ok(hip.hipStreamSynchronize(s2))
+        assert np.array_equal(dY.to_numpy(np.float32, (g.n_rows, N)), want), f"round {rep}, stream 1"
+        assert np.array_equal(dY2.to_numpy(np.float32, (g.n_rows, N)), want2), f"round {rep}, stream 2"
+    # a stream that is gone does not break the next run (the handle waits for the device instead)
     op.run(dX, dY, N, stream=s1.value)
     ok(hip.hipStreamSynchronize(s1))
-    op.run(dX, dY, N, stream=s2.value)                    # the first run has finished: fine
+    ok(hip.hipStreamDestroy(s1))
+    op.run(dX2, dY2, N, stream=s2.value)
     ok(hip.hipStreamSynchronize(s2))
-    for _ in range(300):                                  # some 40 ms of queued work on s1
-        op.run(dX, dY, N, stream=s1.value)
-    with pytest.raises(gpu.AccelError) as e:
-        op.run(dX, dY, N, stream=s2.value)
-    assert e.value.status == gpu._lib.ERR_STATE and "another stream" in e.value.message
-    op.run(dX, dY, N, stream=s1.value)                    # the same stream is always fine
-    ok(hip.hipStreamSynchronize(s1))
-    op.run(dX, dY, N, stream=s2.value)                    # and so is the other one, after the wait
-    ok(hip.hipStreamSynchronize(s2))
-    Y = dY.to_numpy(np.float32, (g.n_rows, N))
-    assert so.check(Y, g.indptr, g.indices, g.values, X) <= so.TOL
+    assert np.array_equal(dY2.to_numpy(np.float32, (g.n_rows, N)), want2)
+    ok(hip.hipStreamDestroy(s2))
+    for b in (dX, dX2, dY, dY2):
+        b.close()
+    op.close()
+
+
+def test_value_update_is_ordered_on_the_device(gpu, hip):
+    """accel_update_values_async queues one kernel and returns: an update and the run behind
+    it need no host wait, on one stream or on two, and give the bits of a fresh operator on
+    the new values; runs queued before the update compute with the old ones."""
+    g = gpu.synthetic.cfg2()
+    N = 64
+    X = gpu.synthetic.dense_operand("cfg2", g.n_cols, N)
+    v0 = np.ascontiguousarray(g.values, dtype=np.float32)
+    v1 = np.random.default_rng(1).uniform(-2, 2, v0.size).astype(np.float32)
+    v2 = np.random.default_rng(2).uniform(-2, 2, v0.size).astype(np.float32)
+
+    def fresh(v):
+        o = gpu.AccelSpMM(g.indptr, g.indices, v, g.n_cols).preprocess()
+        Y = o.matmul(X)
+        o.close()
+        return Y
+
+    want0, want1, want2 = fresh(v0), fresh(v1), fresh(v2)
+    assert so.check(want1, g.indptr, g.indices, v1, X) <= so.TOL
+    op = gpu.AccelSpMM(g.indptr, g.indices, v0, g.n_cols).preprocess()
+    dX = gpu.DeviceBuffer.from_numpy(X)
+    dYa, dYb, dYc = (gpu.DeviceBuffer(g.n_rows * N * 4) for _ in range(3))
+    dV1, dV2 = gpu.DeviceBuffer.from_numpy(v1), gpu.DeviceBuffer.from_numpy(v2)
+    s1, s2 = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(s1)))
+    ok(hip.hipStreamCreate(C.byref(s2)))
+    op.update_values_async(dV1, stream=s1.value)          # the first update builds the position map
+    op.update_values(v0)                                  # back to the old values (host array, waits)
+    free0, free1, total = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    ok(hip.hipDeviceSynchronize())
+    ok(hip.hipMemGetInfo(C.byref(free0), C.byref(total)))
+    for rep in range(3):
+        for d in (dYa, dYb, dYc):
+            d.fill_u32(0x7FC00000)
+        op.synchronize()
+        for _ in range(50):                               # old values, in flight on s1
+            op.run(dX, dYa, N, stream=s1.value)
+        op.update_values_async(dV1, stream=s2.value)      # waits for them on the device
+        op.run(dX, dYb, N, stream=s2.value)               # same stream as the update
+        op.update_values_async(dV2, stream=s2.value)
+        op.run(dX, dYc, N, stream=s1.value)               # another stream than the update
+        ok(hip.hipStreamSynchronize(s1))
+        ok(hip.hipStreamSynchronize(s2))
+        assert np.array_equal(dYa.to_numpy(np.float32, (g.n_rows, N)), want0), f"round {rep}: runs before the update"
+        assert np.array_equal(dYb.to_numpy(np.float32, (g.n_rows, N)), want1), f"round {rep}: update + run, one stream"
+        assert np.array_equal(dYc.to_numpy(np.float32, (g.n_rows, N)), want2), f"round {rep}: update + run, two streams"
+        op.update_values(v0)
+    ok(hip.hipDeviceSynchronize())
+    ok(hip.hipMemGetInfo(C.byref(free1), C.byref(total)))
+    # later updates allocate nothing: the map is 9.6 MB; the runtime's own pools (events, staging for
+    # the host array above) may grow by a 2 MiB chunk
+    assert free0.value - free1.value < (4 << 20)
     ok(hip.hipStreamDestroy(s1))
     ok(hip.hipStreamDestroy(s2))
-    dX.close(); dY.close(); op.close()
+    for b in (dX, dYa, dYb, dYc, dV1, dV2):
+        b.close()
+    op.close()
+
+
+def test_captured_update_and_run_follow_the_values(gpu, hip):
+    """A graph that holds a value update and the run behind it: every replay reads the value
+    array as it is then, so rewriting the array in place between replays is all a caller does
+    (upstream's kernel reads val on every launch, spmm_accel.cu:75)."""
+    g, X, op = make_case(gpu, 36, 48)
+    N = 48
+    assert op.info.n_split_rows > 0
+    dX, dY = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer(g.n_rows * N * 4)
+    dV = gpu.DeviceBuffer.from_numpy(np.ascontiguousarray(g.values, dtype=np.float32))
+    s = C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(s)))
+    # a first update inside a capture is refused: it would have to allocate the position map
+    fresh = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    graph = C.c_void_p()
+    ok(hip.hipStreamBeginCapture(s, 0))
+    with pytest.raises(gpu.AccelError) as e:
+        fresh.update_values_async(dV, stream=s.value)
+    assert e.value.status == gpu._lib.ERR_STATE and "before the capture" in e.value.message
+    hip.hipStreamEndCapture(s, C.byref(graph))
+    if graph.value:
+        hip.hipGraphDestroy(graph)
+    fresh.close()
+    op.update_values_async(dV)                            # outside: builds the map
+    op.run(dX, dY, N)                                     # and the partial-sum buffer
+    op.synchronize()
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamBeginCapture(s, 0))
+    op.update_values_async(dV, stream=s.value)
+    op.run(dX, dY, N, stream=s.value)
+    ok(hip.hipStreamEndCapture(s, C.byref(graph)))
+    ok(hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0))
+    for seed in (1, 2, 3, 4):
+        v = np.random.default_rng(seed).uniform(-1, 1, g.values.size).astype(np.float32)
+        gpu._lib.check(gpu.lib().accel_memcpy_h2d(dV.address, v.ctypes.data, v.nbytes))   # in place
+        dY.fill_u32(0x7FC00000)
+        op.synchronize()
+        ok(hip.hipGraphLaunch(gexec, s))
+        ok(hip.hipStreamSynchronize(s))
+        Y = dY.to_numpy(np.float32, (g.n_rows, N))
+        assert so.check(Y, g.indptr, g.indices, v, X) <= so.TOL, f"replay {seed}"
+        ref = gpu.AccelSpMM(g.indptr, g.indices, v, g.n_cols).preprocess()
+        assert np.array_equal(Y.view(np.uint32), ref.matmul(X).view(np.uint32)), f"replay {seed}: bits"
+        ref.close()
+    ok(hip.hipGraphExecDestroy(gexec))
+    ok(hip.hipGraphDestroy(graph))
+    ok(hip.hipStreamDestroy(s))
+    for b in (dX, dY, dV):
+        b.close()
+    op.close()
 
 
 def test_reserve_before_capture(gpu, hip):
@@ -248,6 +373,42 @@ def test_operands_the_gpu_cannot_use_are_refused(gpu):
     assert so.check(dY.to_numpy(np.float32, (g.n_rows, N)), g.indptr, g.indices, g.values, X) <= so.TOL
     for b in (dX, dY, small):
         b.close()
+    op.close()
+
+
+def test_a_recycled_address_is_checked_again(gpu):
+    """The operand check asks the runtime on every call: after a buffer that passed has been
+    freed and a smaller allocation has taken its address, the same call is refused (a check
+    remembered from the first call would let the kernel run past the new allocation)."""
+    g, X, op = make_case(gpu, 37, 64)
+    N = 64
+    dX = gpu.DeviceBuffer.from_numpy(X)
+    need = g.n_rows * N * 4
+    dY = gpu.DeviceBuffer(need)
+    op.run(dX, dY, N)                                     # passes, with this address and size
+    op.synchronize()
+    addr = dY.address
+    dY.close()
+    small, others = None, []
+    for size in (need - 4096, need // 2, need // 4, need // 16):   # allocators hand freed addresses out again
+        for _ in range(16):
+            b = gpu.DeviceBuffer(size)
+            if b.address == addr:
+                small = b
+                break
+            others.append(b)
+        if small is not None:
+            break
+    for b in others:
+        b.close()
+    if small is None:
+        dX.close(); op.close()
+        pytest.skip("the allocator did not hand the freed address out again")
+    with pytest.raises(gpu.AccelError) as e:
+        op.run(dX, addr, N)
+    assert e.value.status == gpu._lib.ERR_ARG and "allocation holds" in e.value.message
+    small.close()
+    dX.close()
     op.close()
 
 

@@ -53,6 +53,53 @@ def test_same_bits_as_accel_run_twice_second_call_smaller(gpu):
         op_small.close()
 
 
+def test_first_call_on_a_fresh_handle_allocates_nothing(gpu):
+    """The property the entry point exists for: on a handle that has never run (so that no
+    partial-sum buffer exists yet) accel_run_static leaves the free device memory where it
+    was, while the first accel_run afterwards allocates the handle's buffer."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so.7")
+    for name in ("hipMemGetInfo", "hipDeviceSynchronize"):
+        getattr(hip, name).restype = C.c_int
+
+    def free_bytes():
+        assert hip.hipDeviceSynchronize() == 0
+        free, total = C.c_size_t(), C.c_size_t()
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    # 6,000 split rows of 8 column groups each: 48,000 pieces, 24.6 MB of partial sums at N = 128
+    deg = np.concatenate([np.random.default_rng(9).integers(0, 60, 2000), np.full(6000, 400)])
+    g = helpers.graph_from_degrees(deg, n_cols=6000, seed=9)
+    N = 128
+    slack = 2 << 20        # the runtime's own pools move in chunks of this size, in either direction
+    X = np.random.default_rng(15).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    dX = gpu.DeviceBuffer.from_numpy(X)
+    dY = gpu.DeviceBuffer(g.n_rows * N * 4)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess(plan_team=1)
+    try:
+        assert op.info.n_split_rows == 6000
+        dY.fill_u32(0x7FC00000)
+        free_bytes()
+        before = free_bytes()
+        op.run_static(dX, dY, N)                          # the handle's first run of any kind
+        after = free_bytes()
+        assert before - after <= slack, f"accel_run_static took {before - after} bytes of device memory"
+        Y_static = dY.to_numpy(np.float32, (g.n_rows, N))
+        assert so.check(Y_static, g.indptr, g.indices, g.values, X) <= TOL
+        op.run_static(dX, dY, 16)                         # another N: still nothing
+        assert before - free_bytes() <= slack
+        dY.fill_u32(0x7FC00000)
+        now = free_bytes()
+        op.run(dX, dY, N)                                 # accel_run does allocate its buffer (24.6 MB)
+        assert now - free_bytes() >= 6000 * 8 * N * 4 - slack
+        assert np.array_equal(dY.to_numpy(np.float32, (g.n_rows, N)).view(np.uint32), Y_static.view(np.uint32))
+    finally:
+        dX.close()
+        dY.close()
+        op.close()
+
+
 def test_workgroup_units_and_no_split_rows(gpu):
     """Small matrices (a workgroup per unit) and matrices without split rows use no
     scratch at all; the entry point must still give accel_run's result."""
