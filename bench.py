@@ -231,6 +231,7 @@ def main():
     ap.add_argument("--panel", type=int, default=0, help="column-panel width (accel_set_plan_panel; 0 = the library's choice)")
     ap.add_argument("--plan-split", type=int, default=0, help="rows above this many non-zeros are split (accel_set_plan_split; 0 = the library's choice)")
     ap.add_argument("--plan-groups", type=int, default=0, help="column groups of split rows (accel_set_plan_groups; 0 = per row)")
+    ap.add_argument("--plan-reduce", type=int, default=0, help="where split rows are added up (accel_set_plan_reduce; 1 = in the gather kernel, 2 = second kernel, 0 = the library's choice)")
     ap.add_argument("--ld", type=int, default=0,
                     help="also time accel_run_strided with rows of X and Y this many floats apart (>= N), "
                          "on the host clock; reported as config.strided")
@@ -289,7 +290,8 @@ def main():
     t0 = time.time()
     op = pkg.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols)
     t_upload = time.time() - t0
-    plan = {k: v for k, v in (("plan_split", a.plan_split), ("plan_groups", a.plan_groups)) if v}
+    plan = {k: v for k, v in (("plan_split", a.plan_split), ("plan_groups", a.plan_groups),
+                              ("plan_reduce", a.plan_reduce)) if v}
     op.preprocess(**plan)
     first_preprocess_ms = op.info.preprocess_ms      # includes loading the kernels into the GPU
     op.preprocess(**plan)                            # the same work again: what a second graph would cost
@@ -384,7 +386,7 @@ def main():
     achieved = alg_bytes / (main_avg_ms * 1e-3) / 1e9
     achieved_all = alg_bytes / (float(np.mean(tot_ms)) * 1e-3) / 1e9
     profiled, traffic_note = recorded_traffic(a.workload, N)
-    if a.panel or a.plan_split or a.plan_groups:
+    if a.panel or a.plan_split or a.plan_groups or a.plan_reduce:
         profiled, traffic_note = None, "run with plan options: not the configuration that was profiled"
     traffic = profiled.get("traffic_bytes") if profiled else None
     l2_hit_rate = profiled.get("l2_hit_rate") if profiled else None

@@ -39,7 +39,8 @@ class Info(C.Structure):
                 ("n_zero_rows", C.c_int64), ("max_degree", C.c_int32), ("already_sorted", C.c_int32),
                 ("preprocess_ms", C.c_double), ("n_plan_units", C.c_int64), ("n_split_rows", C.c_int64),
                 ("plan_unit_nz", C.c_int32), ("plan_groups", C.c_int32),
-                ("plan_split_nz", C.c_int32), ("plan_team", C.c_int32), ("plan_queues", C.c_int32)]
+                ("plan_split_nz", C.c_int32), ("plan_team", C.c_int32), ("plan_queues", C.c_int32),
+                ("plan_reduce", C.c_int32), ("n_plan_pieces", C.c_int64)]
 
 
 class RunArgs(C.Structure):
@@ -79,6 +80,7 @@ SIGNATURES = {
     "accel_set_plan_team": (C.c_int, [vp, C.c_int]),
     "accel_set_plan_panel": (C.c_int, [vp, C.c_int]),
     "accel_set_plan_queues": (C.c_int, [vp, C.c_int]),
+    "accel_set_plan_reduce": (C.c_int, [vp, C.c_int]),
     "accel_save_state": (C.c_int, [vp, C.c_char_p]),
     "accel_load_state": (C.c_int, [vp, C.c_char_p]),
     "accel_update_values": (C.c_int, [vp, vp, C.c_int]),

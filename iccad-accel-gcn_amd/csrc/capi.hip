@@ -56,7 +56,7 @@ void release_products(accel_handle *h)
     h->writer_done = nullptr; h->writer = nullptr; h->writer_pending = false;
     h->partial_slot = -1; h->next_victim = 0; h->track_runs = false;
     h->perm = nullptr; h->s_indptr = nullptr; h->s_idx = nullptr; h->s_val = nullptr;
-    h->work = nullptr; h->long_slot = nullptr; h->block4 = nullptr; h->partial = nullptr;
+    h->work = nullptr; h->long_slot = nullptr; h->row_done = nullptr; h->block4 = nullptr; h->partial = nullptr;
     h->n_units = h->n_long_units = 0;
     h->partial_floats = 0; h->owns_sorted = false; h->ready = false;
 }
@@ -591,6 +591,19 @@ int accel_set_plan_queues(accel_handle *h, int queues)
     return ACCEL_OK;
 }
 
+int accel_set_plan_reduce(accel_handle *h, int mode)
+{
+    clear_error();
+    if (!h) { set_error("accel_set_plan_reduce: null handle"); return ACCEL_ERR_ARG; }
+    if (mode < 0 || mode > 2) {
+        set_error("accel_set_plan_reduce: mode must be 0 (automatic), 1 (in the gather kernel) or 2 (second "
+                  "kernel), got %d", mode);
+        return ACCEL_ERR_ARG;
+    }
+    h->plan_reduce_option = mode;
+    return ACCEL_OK;
+}
+
 int accel_set_plan_panel(accel_handle *h, int columns)
 {
     clear_error();
@@ -712,6 +725,8 @@ int accel_get_info(const accel_handle *h, accel_info *out)
     out->plan_split_nz = h->plan_split;
     out->plan_team = h->plan_team ? 1 : 0;
     out->plan_queues = h->plan_queues;
+    out->plan_reduce = h->fused_reduce ? 1 : 2;
+    out->n_plan_pieces = h->n_long_units;
     return ACCEL_OK;
 }
 

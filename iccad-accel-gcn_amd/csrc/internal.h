@@ -95,6 +95,10 @@ struct accel_handle {
     int64_t n_units = 0;              // multiple of 4 * plan_queues
     int64_t n_long_units = 0;         // units that write a partial sum
     int32_t *long_slot = nullptr;     // [n_split_rows+1] partial-sum slots of each split row
+    int32_t *row_done = nullptr;      // [n_split_rows] pieces of each split row stored so far in the running
+                                      // launch; zero between launches (part of the long_slot allocation)
+    int plan_reduce_option = 0;       // 0: choose (in the gather kernel); 1: in the gather kernel; 2: second kernel
+    bool fused_reduce = true;         // split rows are added up by the gather kernel itself
     // plan granularity: rows with more than plan_split non-zeros are cut into pieces of at
     // most plan_unit (through partial sums); block4 entries of shorter rows are cut into
     // units of whole rows holding at most plan_unit non-zeros.  384 = one unit per entry.

@@ -1126,6 +1126,17 @@ int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
     return ACCEL_OK;
 }
 
+// Split rows are added up by the gather kernel itself (the wavefront that stores a row's last
+// piece does it: one launch) when the plan holds at most this many pieces, by a second kernel
+// otherwise.  In the kernel every piece ends on a wait for its stores and one atomic, some
+// microseconds of latency that nothing hides on a launch-bound matrix but that is still less
+// than a second launch costs; with many pieces it adds up to more.  Measured, runs queued
+// back to back, in-kernel against second kernel at N = 16 / 64 / 128: 96 pieces (1.9 M
+// non-zeros) 0.88 / 0.94 / 0.96; 5,160 (1.2 M) 0.88 / 0.90 / 0.96; 8,848 (1.6 M) 0.82 / 0.94 /
+// 0.98; 7,760 (2.4 M) 0.99 / 0.96 / 0.98; 68,608 (14 M) 1.01 / 1.02 / 1.02; 144,561 (27 M)
+// 1.24 / 1.08 / 1.09; 0.5 M pieces (115 M non-zeros, nearly every row split) 1.30 at N = 64.
+constexpr int64_t kFusedReduceMaxPieces = 16384;
+
 // The launch plan.  One work unit per wavefront, kWavesPerGroup units per
 // workgroup, as int4 (x, y, z, w):
 //   x <= 384 : whole rows of one block4 entry (degree, first row, first non-zero,
@@ -1171,7 +1182,9 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
     const uint32_t max_key = (uint32_t)((std::max<int64_t>(h->rows, 1) - 1) >> key_shift);
     int cost_shift = 2;                                // total cost = about (nnz + 10 rows) >> shift + units < 2^31
     while ((((int64_t)h->nnz + 10 * h->rows) >> cost_shift) + h->rows >= ((int64_t)1 << 30)) cost_shift++;
-    if ((rc = dslot.alloc(sizeof(int) * (size_t)(n_long + 1)))) return rc;
+    // the slots of each split row, and behind them one counter per split row (zero between launches)
+    if ((rc = dslot.alloc(sizeof(int) * (size_t)(2 * n_long + 1)))) return rc;
+    if ((rc = fill_u32(dslot.as<int>() + n_long + 1, 0u, (size_t)n_long, s))) return rc;
     if (n_long > 0) {
         if ((rc = row_units.alloc(sizeof(int) * (size_t)n_long))) return rc;
         const int64_t n_bins = (int64_t)kPlanBins * n_long;
@@ -1319,6 +1332,8 @@ static int build_work_list(Arena *tmp, accel_handle *h, const int *gcount, const
     h->n_long_units = n_long_units;
     h->work = static_cast<int32_t *>(dwork.release());
     h->long_slot = static_cast<int32_t *>(dslot.release());
+    h->row_done = h->long_slot + n_long + 1;
+    h->fused_reduce = h->plan_reduce_option == 1 || (h->plan_reduce_option == 0 && n_long_units <= kFusedReduceMaxPieces);
     return ACCEL_OK;
 }
 

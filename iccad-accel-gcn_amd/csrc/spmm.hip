@@ -107,6 +107,85 @@ __device__ __forceinline__ void store_vec(float *__restrict__ p, const float (&v
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// Partial sums that another wavefront of the same launch, possibly on another die, adds up
+// (the row's last piece does, see finish_split_row): stored and loaded as relaxed atomics of
+// device scope.  Such a store goes through to memory instead of staying in the die's L2, and
+// such a load does not take a line the die's L2 may hold from before; no cache is written
+// back or invalidated as a whole, which is what a device-scope fence would do on every piece.
+template <int VEC>
+__device__ __forceinline__ void store_partial(float *__restrict__ p, const float (&v)[VEC])
+{
+#pragma unroll
+    for (int i = 0; i < VEC; i++) __hip_atomic_store(p + i, v[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_partial(const float *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// A piece of a split row has stored its partial sums (this thread's stores included).  Counts
+// the piece in; returns true to all T threads of the team (one wavefront, or the workgroup)
+// if it was the row's last one, after which every piece's sums are in memory: each piece
+// waits for its own stores before it counts itself in, and the counter is one memory location.
+// `flag` is a word of LDS of the team's own.  The counter is left at zero for the next launch.
+template <int T>
+__device__ __forceinline__ bool last_piece_of_row(int *__restrict__ counter, int n_pieces, int tid, int *flag)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // this thread's partial sums have arrived
+    if constexpr (T > 64) __syncthreads();                    // ... and those of the other wavefronts
+    if (tid == 0) {
+        const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = before == n_pieces - 1;
+        if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = last;
+    }
+    if constexpr (T > 64) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+    return *flag != 0;
+}
+
+// Adds the nseg partial sums of a split row in slot order and writes the row: T threads
+// (a wavefront or a workgroup), `red` = T floats of LDS of their own.  The columns are
+// covered cw at a time (cw = the power of two <= T that covers N, or T); the T / cw slot
+// groups take every (T / cw)-th slot and their sums are added in group order, so the result
+// does not depend on which piece finished last.
+template <int T>
+__device__ __forceinline__ void finish_split_row(const float *__restrict__ src, int nseg, float *__restrict__ y,
+                                                 int N, int ld, const float *__restrict__ bias, int relu,
+                                                 int tid, float *red)
+{
+    int cw = 1;
+    while (cw < N && cw < T) cw <<= 1;
+    const int sg = T / cw;
+    const int c_in = tid % cw, my_sg = tid / cw;
+    for (int c0 = 0; c0 < N; c0 += cw) {
+        const int c = c0 + c_in;
+        float acc = 0.0f;
+        if (c < N) {
+            int s = my_sg;
+            for (; s + 7 * sg < nseg; s += 8 * sg) {          // eight loads in flight, added in order
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = load_partial(src + (int64_t)(s + u * sg) * ld + c);
+#pragma unroll
+                for (int u = 0; u < 8; u++) acc += v[u];
+            }
+            for (; s < nseg; s += sg) acc += load_partial(src + (int64_t)s * ld + c);
+        }
+        if (sg > 1) {
+            red[tid] = acc;
+            if constexpr (T > 64) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+            if (my_sg == 0)
+                for (int q = 1; q < sg; q++) acc += red[q * cw + c_in];
+            if constexpr (T > 64) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+        }
+        if (my_sg == 0 && c < N) {
+            if (bias) acc += bias[c];
+            if (relu) acc = fmaxf(acc, 0.0f);
+            y[c] = acc;
+        }
+    }
+}
+
 // One lane group's share of one row: non-zeros k, k + gp, ... of the d pairs at row_st are
 // multiplied with their rows of X and added into acc.  U gathers are issued back to back;
 // full batches carry no masks, only the last batch of a row is predicated.
@@ -196,7 +275,8 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
     const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
     const int32_t *__restrict__ perm, const float *__restrict__ X, float *__restrict__ Y,
     float *__restrict__ partial, int N, int ld, int n_zero_rows, int n_zero_groups,
-    const float *__restrict__ bias, int relu)
+    const float *__restrict__ bias, int relu, const int32_t *__restrict__ long_slot, int first_split_row,
+    int *__restrict__ row_done)
 {
     // N columns are computed; rows of X, Y and the partial sums are ld floats apart
     // (ld > N when the launch covers one column panel of a wider operand)
@@ -285,8 +365,9 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
             const int64_t out_row = __shfl(my_out, r < n_rows ? r : 0);
             if (live && k == 0) {
                 if (is_long) {
-                    store_vec<VEC, kShift>(partial + (int64_t)(deg - (kDegBound + 1)) * ld + col, acc,
-                                           streaming);
+                    float *p = partial + (int64_t)(deg - (kDegBound + 1)) * ld + col;
+                    if (row_done) store_partial<VEC>(p, acc);
+                    else store_vec<VEC, kShift>(p, acc, streaming);
                 } else {
                     if (bias) {
 #pragma unroll
@@ -299,6 +380,18 @@ __global__ __launch_bounds__(kWgThreads) void spmm_gather_kernel(
                     store_vec<VEC, kShift>(Y + out_row * ld + col, acc, streaming);
                 }
             }
+        }
+    }
+    // The wavefront that stores a split row's last piece adds the row up, in this launch
+    // (row_done: one counter per split row; null: a second kernel does it).
+    if (is_long && row_done) {
+        const int lr = row0 - first_split_row;
+        const int first = long_slot[lr], nseg = long_slot[lr + 1] - first;
+        int *flag = reinterpret_cast<int *>(st);             // the staged pairs are no longer needed
+        if (last_piece_of_row<64>(row_done + lr, nseg, lane, flag)) {
+            const int64_t out_row = perm ? perm[row0] : row0;
+            finish_split_row<64>(partial + (int64_t)first * ld, nseg, Y + out_row * ld, N, ld, bias, relu, lane,
+                                 reinterpret_cast<float *>(st) + 64);
         }
     }
 }
@@ -314,7 +407,8 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
     const int32_t *__restrict__ s_idx, const float *__restrict__ s_val,
     const int32_t *__restrict__ perm, const float *__restrict__ X, float *__restrict__ Y,
     float *__restrict__ partial, int N, int ld, int n_zero_rows, int n_zero_groups,
-    const float *__restrict__ bias, int relu)
+    const float *__restrict__ bias, int relu, const int32_t *__restrict__ long_slot, int first_split_row,
+    int *__restrict__ row_done)
 {
     constexpr int G = 64 / L;        // lane groups per wavefront
     constexpr int TG = G * kWaves;   // lane groups per workgroup
@@ -413,9 +507,11 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
             }
             const int64_t out_row = __shfl(my_out, r < n_rows ? r : 0);
             if (live && k == 0) {
-                if (is_long)
-                    store_vec<VEC, kShift>(partial + (int64_t)(deg - (kDegBound + 1)) * ld + col, acc, false);
-                else {
+                if (is_long) {
+                    float *p = partial + (int64_t)(deg - (kDegBound + 1)) * ld + col;
+                    if (row_done) store_partial<VEC>(p, acc);
+                    else store_vec<VEC, kShift>(p, acc, false);
+                } else {
                     if (bias) {
 #pragma unroll
                         for (int v = 0; v < VEC; v++) acc[v] += bias[col + v];
@@ -427,6 +523,18 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
                     store_vec<VEC, kShift>(Y + out_row * ld + col, acc, N * 4 >= kStreamingMinBytes);
                 }
             }
+        }
+    }
+    // the workgroup that stores a split row's last piece adds the row up (see the gather kernel)
+    if (is_long && row_done) {                       // workgroup-uniform
+        const int lr = row0 - first_split_row;
+        const int first = long_slot[lr], nseg = long_slot[lr + 1] - first;
+        __syncthreads();                             // every wavefront is done with the staged pairs
+        int *flag = reinterpret_cast<int *>(stage);
+        if (last_piece_of_row<kWgThreads>(row_done + lr, nseg, (int)threadIdx.x, flag)) {
+            const int64_t out_row = perm ? perm[row0] : row0;
+            finish_split_row<kWgThreads>(partial + (int64_t)first * ld, nseg, Y + out_row * ld, N, ld, bias, relu,
+                                         (int)threadIdx.x, reinterpret_cast<float *>(stage) + 64);
         }
     }
 }
@@ -512,6 +620,9 @@ struct LaunchArgs {
     int N, ld, n_zero_rows, n_zero_groups;
     const float *bias;
     int relu;
+    const int32_t *long_slot;
+    int first_split_row;
+    int *row_done;
     // events bound to this launch itself (its start and its end), or null: unlike an event
     // recorded behind the launch they put no packet of their own into the queue
     hipEvent_t start_ev, stop_ev;
@@ -524,21 +635,23 @@ void launch_one(const LaunchArgs &a)
         if (a.team)
             hipExtLaunchKernelGGL((spmm_team_kernel<L, VEC, kWide, kShift>), a.grid, dim3(kWgThreads), 0, a.stream,
                                   a.start_ev, a.stop_ev, 0, a.work, a.n_units, a.s_idx, a.s_val, a.perm, a.X, a.Y,
-                                  a.partial, a.N, a.ld, a.n_zero_rows, a.n_zero_groups, a.bias, a.relu);
+                                  a.partial, a.N, a.ld, a.n_zero_rows, a.n_zero_groups, a.bias, a.relu, a.long_slot,
+                                  a.first_split_row, a.row_done);
         else
             hipExtLaunchKernelGGL((spmm_gather_kernel<L, VEC, kWide, kShift>), a.grid, dim3(kWgThreads), 0, a.stream,
                                   a.start_ev, a.stop_ev, 0, a.work, a.n_units, a.s_idx, a.s_val, a.perm, a.X, a.Y,
-                                  a.partial, a.N, a.ld, a.n_zero_rows, a.n_zero_groups, a.bias, a.relu);
+                                  a.partial, a.N, a.ld, a.n_zero_rows, a.n_zero_groups, a.bias, a.relu, a.long_slot,
+                                  a.first_split_row, a.row_done);
         return;
     }
     if (a.team)
         spmm_team_kernel<L, VEC, kWide, kShift><<<a.grid, dim3(kWgThreads), 0, a.stream>>>(
             a.work, a.n_units, a.s_idx, a.s_val, a.perm, a.X, a.Y, a.partial, a.N, a.ld, a.n_zero_rows,
-            a.n_zero_groups, a.bias, a.relu);
+            a.n_zero_groups, a.bias, a.relu, a.long_slot, a.first_split_row, a.row_done);
     else
         spmm_gather_kernel<L, VEC, kWide, kShift><<<a.grid, dim3(kWgThreads), 0, a.stream>>>(
             a.work, a.n_units, a.s_idx, a.s_val, a.perm, a.X, a.Y, a.partial, a.N, a.ld, a.n_zero_rows,
-            a.n_zero_groups, a.bias, a.relu);
+            a.n_zero_groups, a.bias, a.relu, a.long_slot, a.first_split_row, a.row_done);
 }
 
 // Lane-group widths: 1..64 lanes of one 16-byte vector each; scalar lanes only serve N < 4.
@@ -689,7 +802,10 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     // last waits for that stream on the device (runs queued on one stream are ordered anyway).
     hipEvent_t run_done = nullptr;                  // to be bound to the run's last kernel
     if (int rc = order_run(h, stream, uses_handle_partial, capturing, &run_done)) return rc;
-    const bool has_reduce = h->n_split_rows > 0;
+    // split rows are added up by the gather kernel itself (the wavefront that stores a row's
+    // last piece), or, when the handle has no counters for that, by a second kernel
+    int *row_done = h->fused_reduce ? h->row_done : nullptr;
+    const bool has_reduce = h->n_split_rows > 0 && !row_done;
     // Wide operands are computed one column panel at a time (all units for the first
     // panel, then all units for the next): a panel's slice of X is what the L2s have
     // to hold, and a narrower slice means more rows of X fit.
@@ -731,6 +847,7 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         if (last && !stop && !has_reduce) stop = run_done;      // the run ends with this launch
         const LaunchArgs la{h->plan_team, grid, stream, wk, (int)h->n_units, h->s_idx, h->s_val, h->perm,
                             Xp, Yp, Pp, n, ld, (int)h->n_zero_rows, (int)zero_groups, bp, relu,
+                            h->long_slot, (int)(h->rows - h->n_split_rows), row_done,
                             first ? main_start : nullptr, stop};
         const int rc = launch_for_mode(mode, wide, L, la);
         if (rc) return rc;

@@ -35,7 +35,7 @@ struct StateHeader {
     int32_t identity_perm;            // 1: the rows were already in degree order, no permutation follows
     int64_t rows, cols, nnz;
     int32_t plan_unit_option, plan_split_option, plan_groups, plan_team_option, plan_queues_option;
-    int32_t reserved;
+    int32_t plan_reduce_option;
     int64_t perm_words;               // rows, or 0 with identity_perm
     uint64_t header_hash;             // FNV-1a of this header with header_hash = 0
 };
@@ -97,6 +97,7 @@ int accel_save_state(const accel_handle *h, const char *path)
     hd.plan_unit_option = h->plan_unit_option; hd.plan_split_option = h->plan_split_option;
     hd.plan_groups = h->plan_groups; hd.plan_team_option = h->plan_team_option;
     hd.plan_queues_option = h->plan_queues_option;
+    hd.plan_reduce_option = h->plan_reduce_option;
     hd.perm_words = h->identity_perm ? 0 : h->rows;
     hd.header_hash = header_hash(hd);
     PinnedBuf host;
@@ -163,7 +164,8 @@ int accel_load_state(accel_handle *h, const char *path)
                       (hd.plan_groups == 0 || hd.plan_groups == 8 || hd.plan_groups == 16 ||
                        hd.plan_groups == 32 || hd.plan_groups == 64) &&
                       hd.plan_team_option >= 0 && hd.plan_team_option <= 2 &&
-                      (hd.plan_queues_option == 0 || hd.plan_queues_option == 1 || hd.plan_queues_option == kXcds);
+                      (hd.plan_queues_option == 0 || hd.plan_queues_option == 1 || hd.plan_queues_option == kXcds) &&
+                      hd.plan_reduce_option >= 0 && hd.plan_reduce_option <= 2;
     if (!sane) { set_error("%s: inconsistent header", path); return ACCEL_ERR_META; }
     // the file must be exactly as long as the header says, before anything is allocated from it
     {
@@ -198,17 +200,18 @@ int accel_load_state(accel_handle *h, const char *path)
     release_products(h);
     // the options of the state replace the handle's, so that the handle ends up as the one
     // that was saved; they come back if the load fails
-    const int keep[5] = {h->plan_unit_option, h->plan_split_option, h->plan_groups, h->plan_team_option,
-                         h->plan_queues_option};
+    const int keep[6] = {h->plan_unit_option, h->plan_split_option, h->plan_groups, h->plan_team_option,
+                         h->plan_queues_option, h->plan_reduce_option};
     h->plan_unit_option = hd.plan_unit_option; h->plan_split_option = hd.plan_split_option;
     h->plan_groups = hd.plan_groups; h->plan_team_option = hd.plan_team_option;
     h->plan_queues_option = hd.plan_queues_option;
+    h->plan_reduce_option = hd.plan_reduce_option;
     const int rc = preprocess_device(h, &order);
     (void)hipStreamSynchronize(nullptr);            // the staging buffers go away with this scope
     if (rc) {
         release_products(h);
         h->plan_unit_option = keep[0]; h->plan_split_option = keep[1]; h->plan_groups = keep[2];
-        h->plan_team_option = keep[3]; h->plan_queues_option = keep[4];
+        h->plan_team_option = keep[3]; h->plan_queues_option = keep[4]; h->plan_reduce_option = keep[5];
         return rc;
     }
     h->preprocess_ms =

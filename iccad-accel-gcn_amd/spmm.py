@@ -61,14 +61,17 @@ class AccelSpMM:
     # -- preprocess ---------------------------------------------------------
     def preprocess(self, plan_unit: int | None = None, plan_groups: int | None = None,
                    plan_split: int | None = None, plan_team: int | None = None,
-                   plan_queues: int | None = None) -> "AccelSpMM":
+                   plan_queues: int | None = None, plan_reduce: int | None = None) -> "AccelSpMM":
         """Degree sort, block4 metadata and launch plan on the GPU.  ``plan_unit``
         (16..384) overrides the automatic choice of non-zeros per unit,
         ``plan_groups`` (8, 16, 32, 64) that of column groups for split rows,
         ``plan_split`` (16..384) the row length above which rows are split,
         ``plan_team`` (1: one wavefront per unit, 2: one workgroup per unit) who
         works on a unit, ``plan_queues`` (8 or 1) the number of interleaved queues of
-        the plan (default: from the shape of the device)."""
+        the plan (default: from the shape of the device), ``plan_reduce`` (1: the gather
+        kernel adds split rows up itself, 2: a second kernel does) where partial sums meet."""
+        if plan_reduce is not None:
+            check(lib().accel_set_plan_reduce(self._h, int(plan_reduce)))
         if plan_queues is not None:
             check(lib().accel_set_plan_queues(self._h, int(plan_queues)))
         if plan_team is not None:

@@ -195,6 +195,18 @@ int accel_update_values_async(accel_handle *h, const float *val_dev, void *strea
  * before accel_preprocess; accel_info.plan_queues tells what was used. */
 int accel_set_plan_queues(accel_handle *h, int queues);
 
+/* Where the partial sums of split rows are added up.  Upstream's run is one launch
+ * (spmm_accel.cu:104-108) whose blocks add long rows into vout with atomicAdd (:84,97).
+ * Here every piece of a split row stores its sum to a slot of its own and the slots are
+ * added in a fixed order (results are the same bits on every run): 1 = by the gather
+ * kernel itself, one launch: each piece counts itself in on a per-row counter and the
+ * wavefront that stores the row's last piece adds the row up; 2 = by a second, small
+ * kernel behind the gather kernel; 0 (the default) = the library chooses: 1 when the
+ * plan holds at most 16,384 pieces (launch-bound matrices, where a second launch costs
+ * more than the wait each piece then ends on), 2 otherwise.
+ * Call before accel_preprocess. */
+int accel_set_plan_reduce(accel_handle *h, int mode);
+
 /* Column panels (no counterpart upstream, which always walks all N columns of a row
  * at once, spmm_accel.cu:37-48): one accel_run computes Y one panel of `columns`
  * columns at a time (the last one narrower when N is not a multiple), all work units
@@ -224,6 +236,8 @@ typedef struct accel_info {
     int32_t plan_split_nz;  /* rows with more non-zeros than this are cut into pieces */
     int32_t plan_team;      /* 1: a unit is worked on by a whole workgroup, 0: by one wavefront */
     int32_t plan_queues;    /* interleaved queues of the launch plan: 8 (one per die) or 1 */
+    int32_t plan_reduce;    /* 1: the gather kernel adds split rows up itself, 2: a second kernel does */
+    int64_t n_plan_pieces;  /* units of the plan that are pieces of split rows (each has a partial-sum slot) */
 } accel_info;
 int accel_get_info(const accel_handle *h, accel_info *out);
 
