@@ -410,7 +410,9 @@ def main():
                    "reference_protocol_ms": round(ref_protocol_ms, 5),
                    "ms_per_step_without_events": round(ms_per_step_no_events, 5),
                    "plan": {"split_nz": int(info.plan_split_nz), "groups": int(info.plan_groups),
-                            "unit_nz": int(info.plan_unit_nz), "panel": a.panel}},
+                            "unit_nz": int(info.plan_unit_nz), "panel": a.panel,
+                            "queues": int(info.plan_queues), "pieces": int(info.n_plan_pieces),
+                            "split_rows_added_up": "in the gather kernel" if info.plan_reduce == 1 else "by a second kernel"}},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": traffic,

@@ -543,13 +543,17 @@ __global__ __launch_bounds__(kWgThreads) void spmm_team_kernel(
 // The first n_shared_groups workgroups take rpw rows each (256 / rpw threads per
 // row): rows with few slots and few columns do not need a whole workgroup.  The
 // remaining workgroups take one row each: the rows with very many slots.
+// A thread covers VEC consecutive columns (VEC = 4: one 16-byte load per slot, when N and
+// the row stride are multiples of 4 and the operands 16-byte aligned; else VEC = 1); NV = the
+// row's columns counted in such vectors.
+template <int VEC>
 __global__ __launch_bounds__(kReduceThreads) void long_row_reduce_kernel(
     const float *__restrict__ partial, const int32_t *__restrict__ long_slot,
     const int32_t *__restrict__ perm, int64_t first_split_row, int n_shared_rows, int n_shared_groups,
-    int rpw, int n_rows, float *__restrict__ Y, int N, int ld, const float *__restrict__ bias, int relu)
+    int rpw, int n_rows, float *__restrict__ Y, int NV, int ld, const float *__restrict__ bias, int relu)
 {
-    // N columns; rows of Y and of the partial sums are ld floats apart
-    __shared__ float red[kReduceThreads];
+    // rows of Y and of the partial sums are ld floats apart
+    __shared__ float red[kReduceThreads][VEC];
     const bool shared_group = (int)blockIdx.x < n_shared_groups;
     const int T = shared_group ? kReduceThreads / rpw : kReduceThreads;   // threads per row
     const int sub_row = threadIdx.x / T, t = threadIdx.x % T;
@@ -561,34 +565,55 @@ __global__ __launch_bounds__(kReduceThreads) void long_row_reduce_kernel(
     const float *src = partial + (int64_t)first * ld;
     const int64_t r = first_split_row + lr;
     const int64_t out_row = row_ok ? (perm ? perm[r] : r) : 0;
-    int cw = 1;                                    // columns per pass: power of two <= T
-    while (cw < N && cw < T) cw <<= 1;
+    int cw = 1;                                    // vectors per pass: power of two <= T
+    while (cw < NV && cw < T) cw <<= 1;
     const int sg = T / cw;                         // slot groups
     const int c_in = t % cw, my_sg = t / cw;
-    for (int c0 = 0; c0 < N; c0 += cw) {
-        const int c = c0 + c_in;
-        float acc = 0.0f;
-        if (c < N) {
+    for (int c0 = 0; c0 < NV; c0 += cw) {
+        const int c = (c0 + c_in) * VEC;           // first column of this thread's vector
+        const bool col_ok = c0 + c_in < NV;
+        float acc[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[v] = 0.0f;
+        if (col_ok) {
             int sgm = my_sg;
             for (; sgm + 7 * sg < nseg; sgm += 8 * sg) {       // eight loads in flight, added in order
-                float v[8];
+                float x[8][VEC];
 #pragma unroll
-                for (int u = 0; u < 8; u++) v[u] = src[(int64_t)(sgm + u * sg) * ld + c];
+                for (int u = 0; u < 8; u++) load_vec<VEC, false>(src + (int64_t)(sgm + u * sg) * ld + c, x[u]);
 #pragma unroll
-                for (int u = 0; u < 8; u++) acc += v[u];
+                for (int u = 0; u < 8; u++)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[v] += x[u][v];
             }
-            for (; sgm < nseg; sgm += sg) acc += src[(int64_t)sgm * ld + c];
+            for (; sgm < nseg; sgm += sg) {
+                float x[VEC];
+                load_vec<VEC, false>(src + (int64_t)sgm * ld + c, x);
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[v] += x[v];
+            }
         }
-        red[threadIdx.x] = acc;
-        __syncthreads();
-        if (row_ok && my_sg == 0 && c < N) {
-            float sum = acc;
-            for (int q = 1; q < sg; q++) sum += red[sub_row * T + q * cw + c_in];
-            if (bias) sum += bias[c];
-            if (relu) sum = fmaxf(sum, 0.0f);
-            Y[out_row * ld + c] = sum;
+        if (sg > 1) {                              // uniform over the workgroup's rows of one kind
+#pragma unroll
+            for (int v = 0; v < VEC; v++) red[threadIdx.x][v] = acc[v];
+            __syncthreads();
+            if (my_sg == 0)
+                for (int q = 1; q < sg; q++)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[v] += red[sub_row * T + q * cw + c_in][v];
+            __syncthreads();
         }
-        __syncthreads();
+        if (row_ok && my_sg == 0 && col_ok) {
+            if (bias) {
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[v] += bias[c + v];
+            }
+            if (relu) {
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[v] = fmaxf(acc[v], 0.0f);
+            }
+            store_vec<VEC, false>(Y + out_row * ld + c, acc, false);
+        }
     }
 }
 
@@ -856,20 +881,26 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
         ACCEL_HIP(hipEventRecord(run_done, stream));
     if (has_reduce) {
         // one launch: rows with very many slots (the last n_big rows) get a workgroup each, the
-        // others share one between 4, 2 or 1 rows depending on how many threads N can use
+        // others share one: as many rows per workgroup as leaves a row one thread per vector
+        // of columns (16 at least, so that a row's loads stay coalesced)
         const int n_split = (int)h->n_split_rows, n_big = (int)h->n_big_rows, n_shared = n_split - n_big;
-        const int rpw = N <= 64 ? 4 : N <= 128 ? 2 : 1;
+        const int rvec = mode == 0 ? 4 : 1;          // 16-byte accesses need the same as the gather kernel's
+        const int nv = (N + rvec - 1) / rvec;
+        int threads_per_row = 16;
+        while (threads_per_row < nv && threads_per_row < kReduceThreads) threads_per_row <<= 1;
+        const int rpw = kReduceThreads / threads_per_row;
         const int shared_groups = (n_shared + rpw - 1) / rpw;
         const dim3 rgrid((unsigned)(shared_groups + n_big));
+        auto kernel = rvec == 4 ? long_row_reduce_kernel<4> : long_row_reduce_kernel<1>;
         if (run_done)
-            hipExtLaunchKernelGGL(long_row_reduce_kernel, rgrid, dim3(kReduceThreads), 0, stream, nullptr, run_done,
+            hipExtLaunchKernelGGL(kernel, rgrid, dim3(kReduceThreads), 0, stream, nullptr, run_done,
                                   0, (const float *)partial, (const int32_t *)h->long_slot, (const int32_t *)h->perm,
-                                  (int64_t)(h->rows - h->n_split_rows), n_shared, shared_groups, rpw, n_split, Y, N,
+                                  (int64_t)(h->rows - h->n_split_rows), n_shared, shared_groups, rpw, n_split, Y, nv,
                                   ld, bias, relu);
         else
-            long_row_reduce_kernel<<<rgrid, dim3(kReduceThreads), 0, stream>>>(
+            kernel<<<rgrid, dim3(kReduceThreads), 0, stream>>>(
                 partial, h->long_slot, h->perm, h->rows - h->n_split_rows, n_shared, shared_groups, rpw,
-                n_split, Y, N, ld, bias, relu);
+                n_split, Y, nv, ld, bias, relu);
     }
     ACCEL_HIP(hipGetLastError());
     return ACCEL_OK;
