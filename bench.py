@@ -204,7 +204,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--warmup", type=int, default=40,
+                    help="untimed steps before the timed ones; the GPU reaches its steady clocks after some "
+                         "60 ms of load (about 19 steps of the default workload run 4 %% slower than all later ones)")
     ap.add_argument("--workload", default="cfg4",
                     help="cfg1..cfg5, or fixture:<name> for the degree sequence of one of the "
                          "reference's graphs (e.g. fixture:OVCAR-8H, fixture:ppa) with uniform random "

@@ -98,6 +98,15 @@ def build_cli(verbose: bool = False) -> Path:
         r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed for {name}.cpp:\n" + r.stdout)
+    # a driver written the way upstream's main.cu is, against include/ alone (run by the tests)
+    caller = ROOT / "tests" / "cases" / "upstream_shaped_caller.cpp"
+    if caller.exists():
+        cmd = [hipcc(), "-x", "hip", f"--offload-arch={ARCH}", "-O2", "-std=c++17", "-Wno-unused-value",
+               f"-I{ROOT / 'include'}", str(caller), "-o", str(BIN_DIR / "upstream_shaped_caller"),
+               f"-L{LIB_DIR}", "-laccelgcn", "-Wl,-rpath,$ORIGIN/../lib"]
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed for upstream_shaped_caller.cpp:\n" + r.stdout)
     return BIN_DIR / "spmm_test"
 
 

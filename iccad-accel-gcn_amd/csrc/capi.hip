@@ -46,6 +46,7 @@ void release_products(accel_handle *h)
     if (h->partial) (void)hipFree(h->partial);
     if (h->src_pos) (void)hipFree(h->src_pos);
     h->src_pos = nullptr;
+    h->val_stale = false;
     // what other streams still hold was queued against the memory freed above (hipFree waits
     // for the device), so the bookkeeping starts afresh
     if (h->writer_done) (void)hipEventDestroy(h->writer_done);
@@ -621,6 +622,10 @@ int accel_preprocess(accel_handle *h)
 {
     clear_error();
     if (!h) { set_error("accel_preprocess: null handle"); return ACCEL_ERR_ARG; }
+    if (h->val_stale) {                     // value updates since: the handle's copy of the values first
+        if (hipDeviceSynchronize() != hipSuccess) (void)hipGetLastError();
+        if (int rc = restore_own_values(h, nullptr)) return rc;
+    }
     release_products(h);
     const int rc = preprocess_device(h);
     if (rc) release_products(h);
@@ -642,17 +647,19 @@ static int update_values_on_stream(accel_handle *h, const float *val_dev, hipStr
         if (int rc = build_source_positions(h, stream)) return rc;
     }
     if (int rc = order_update(h, stream, capturing)) return rc;
-    if (h->owns_input) {
-        // the handle's own copy of the caller's values follows (a later accel_preprocess reads it)
+    if (!h->owns_input) h->val = val_dev;   // borrowed from now on (it may be the same array, rewritten)
+    if (h->owns_sorted) {
+        // one kernel: the new values into the sorted copy.  A handle's own copy of the caller's
+        // order is not rewritten here; it is brought back from the sorted copy if a new
+        // preprocessing of the handle ever needs it (restore_own_values).
+        if (int rc = gather_values(h, val_dev, stream)) return rc;
+        if (h->owns_input && val_dev != h->val) h->val_stale = true;
+    } else if (h->owns_input) {
+        // the kernels read the handle's copy of the caller's order in place
         if (val_dev != h->val)
             if (int rc = copy_u32(const_cast<float *>(h->val), val_dev, (size_t)h->nnz, stream)) return rc;
     } else {
-        h->val = val_dev;                   // borrowed from now on (it may be the same array, rewritten)
-    }
-    if (h->owns_sorted) {
-        if (int rc = gather_values(h, h->val, stream)) return rc;
-    } else {
-        h->s_val = h->val;                  // the kernels read the caller's order in place
+        h->s_val = h->val;                  // the kernels read the caller's array in place
     }
     return note_update(h, stream, capturing);
 }
@@ -705,6 +712,7 @@ int accel_update_values(accel_handle *h, const float *val, int flags)
     if (int rc = update_values_on_stream(h, val, s, "accel_update_values")) return rc;
     ACCEL_HIP(hipStreamSynchronize(s));
     h->writer_pending = false;
+    if (flags == ACCEL_PTR_HOST) h->val_stale = false;   // the handle's copy was written first
     return ACCEL_OK;
 }
 

@@ -126,6 +126,9 @@ struct accel_handle {
     size_t partial_floats = 0;
     // sorted position -> position in the caller's arrays, built by the first value update
     int32_t *src_pos = nullptr;
+    // the handle's own copy of the caller's values (owns_input) is behind the sorted copy: a value
+    // update from a device array went into the sorted copy only (restore_own_values brings it back)
+    bool val_stale = false;
     // Which streams use the handle's mutable device memory (see order_run / order_update in
     // capi.hip).  Runs read the sorted values and, with split rows, write and read `partial`;
     // a value update rewrites the sorted values.  A tracked run leaves an event, bound to its
@@ -154,6 +157,7 @@ struct SavedOrder {               // a degree-sort order read from a saved state
 int preprocess_device(accel_handle *h, const SavedOrder *given = nullptr);
 int build_source_positions(accel_handle *h, hipStream_t s);
 int gather_values(accel_handle *h, const float *val, hipStream_t s);
+int restore_own_values(accel_handle *h, hipStream_t s);
 // capi.hip
 void release_products(accel_handle *h);
 bool stream_is_capturing(hipStream_t s);

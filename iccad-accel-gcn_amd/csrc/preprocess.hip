@@ -1447,6 +1447,40 @@ int gather_values(accel_handle *h, const float *val, hipStream_t s)
     return ACCEL_OK;
 }
 
+// The other direction: val[src_pos[p]] = s_val[p].  A handle that owns a copy of the caller's
+// values lets that copy go stale when the values are updated from a device array (the update
+// then is the one gather above); the copy is only read again by a new preprocessing of the
+// same handle, which calls this first.  Synchronises s.
+__global__ __launch_bounds__(kThreads) void scatter_values_kernel(const float *__restrict__ s_val,
+                                                                  const int32_t *__restrict__ src_pos,
+                                                                  float *__restrict__ val, int64_t nnz)
+{
+    const int64_t p = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 4;
+    if (p + 4 <= nnz) {
+        const int4 q = *reinterpret_cast<const int4 *>(src_pos + p);
+        const float4 v = *reinterpret_cast<const float4 *>(s_val + p);
+        val[q.x] = v.x; val[q.y] = v.y; val[q.z] = v.z; val[q.w] = v.w;
+    } else {
+        for (int64_t i = p; i < nnz; i++) val[src_pos[i]] = s_val[i];
+    }
+}
+
+int restore_own_values(accel_handle *h, hipStream_t s)
+{
+    if (!h->val_stale) return ACCEL_OK;
+    if (!h->owns_input || !h->owns_sorted || !h->src_pos || !h->s_val) {
+        set_error("internal: the handle's copy of the values is stale and cannot be restored");
+        return ACCEL_ERR_STATE;
+    }
+    const int64_t threads = (h->nnz + 3) / 4;
+    scatter_values_kernel<<<dim3(grid_for(threads)), dim3(kThreads), 0, s>>>(
+        h->s_val, h->src_pos, const_cast<float *>(h->val), h->nnz);
+    ACCEL_HIP(hipGetLastError());
+    ACCEL_HIP(hipStreamSynchronize(s));
+    h->val_stale = false;
+    return ACCEL_OK;
+}
+
 // A row order that comes from a saved state is taken only if it is the order the sort would
 // produce: ascending degree, ties by ascending row id.  That order is unique, so checking
 // that the pairs (degree, row) strictly increase along it and that every entry is a row

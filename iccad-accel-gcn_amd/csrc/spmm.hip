@@ -798,7 +798,8 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     float *partial = h->partial;
     const bool uses_handle_partial = !static_partial && h->n_long_units > 0;
     // the capture status is only needed where something depends on it
-    const bool capturing = (uses_handle_partial || h->writer_pending) && stream_is_capturing(stream);
+    const bool capturing =
+        (uses_handle_partial || h->writer_pending || h->track_runs) && stream_is_capturing(stream);
     if (static_partial) {
         partial = nullptr;
         const size_t need = (size_t)h->n_long_units * (size_t)ld;

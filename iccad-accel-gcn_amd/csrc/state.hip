@@ -197,6 +197,10 @@ int accel_load_state(accel_handle *h, const char *path)
         ACCEL_HIP(hipMemcpyAsync(dev.p, host.p, bytes, hipMemcpyHostToDevice, nullptr));
         order.perm_dev = static_cast<const uint32_t *>(dev.p);
     }
+    if (h->val_stale) {                     // value updates since: the handle's copy of the values first
+        if (hipDeviceSynchronize() != hipSuccess) (void)hipGetLastError();
+        if (int rc = restore_own_values(h, nullptr)) return rc;
+    }
     release_products(h);
     // the options of the state replace the handle's, so that the handle ends up as the one
     // that was saved; they come back if the load fails

@@ -170,9 +170,10 @@ int accel_load_state(accel_handle *h, const char *path);
  * streams behind it, so "update, then run" needs no host synchronisation whatever the
  * streams are.  It can be captured into a HIP graph together with the runs that follow
  * (after one update outside the capture has built the map; a capturing stream is only
- * ordered against itself).  A handle that uploaded its CSR also copies the values into
- * its own array (same stream); a handle that borrows device arrays borrows val_dev from
- * now on (it may be the same array, rewritten in place).
+ * ordered against itself).  A handle that borrows device arrays borrows val_dev from now
+ * on (it may be the same array, rewritten in place); a handle that uploaded its CSR keeps
+ * its own copy of the caller's order, which it brings up to date from the sorted copy only
+ * if the handle is preprocessed again.
  *
  * accel_update_values: the same for an array in host memory (ACCEL_PTR_HOST: copied to the
  * device first; only for handles that own their CSR) or on the device (ACCEL_PTR_DEVICE),

@@ -1,13 +1,18 @@
 // A benchmark driver written the way upstream's is (main.cu:1-16 for the includes and the
 // globals, :62-65 for the four graph files, :131 for the constructor, :146 and :166 for the
-// two do_test calls), in this repository's own words.  tests/test_host_abi.py compiles it
-// against include/ to show that such a caller needs nothing beyond those headers: it names
-// `string` before its own using-directive, as upstream does, and uses the host-clock helpers.
+// two do_test calls, :18-51 for the check), in this repository's own words.  It names
+// `string` before its own using-directive, as upstream does, and uses the host-clock helpers
+// and the file readers of the headers.  tests/test_host_abi.py compiles and links it against
+// include/ and the library alone; the build puts it in bin/ and tests/test_cli.py runs it on
+// the GPU on a dataset in upstream's layout.
+//
+//   upstream_shaped_caller <graph> <dim> [natural]     reads ../graphs/<graph>.*
 #include <iostream>
 #include "data.h"
 #include "spmm_accel.h"
 #include <random>
 #include <algorithm>
+#include <vector>
 
 string graph_dir = "../graphs/";
 
@@ -24,34 +29,64 @@ static double mean_abs_diff(const vector<float> &a, const vector<float> &b)
 
 int run_graph(string graph, bool natural_order)
 {
-    int *ptr, *idx;
-    int v_num = natural_order ? hip_read_array(&ptr, graph_dir + graph + ".graph.ptrdump") - 1
-                              : hip_read_array(&ptr, graph_dir + graph + ".new_indptr") - 1;
-    int e_num = natural_order ? hip_read_array(&idx, graph_dir + graph + ".graph.edgedump")
-                              : hip_read_array(&idx, graph_dir + graph + ".new_indices");
-    if (v_num < 0 || e_num < 0) return 1;
+    // the CSR on the device for the operator, and on the host for the check
+    int *ptr, *idx, *h_ptr, *h_idx;
+    string ptr_file = graph_dir + graph + (natural_order ? ".graph.ptrdump" : ".new_indptr");
+    string idx_file = graph_dir + graph + (natural_order ? ".graph.edgedump" : ".new_indices");
+    int v_num = hip_read_array(&ptr, ptr_file) - 1;
+    int e_num = hip_read_array(&idx, idx_file);
+    if (v_num < 0 || e_num < 0 || read_array(&h_ptr, ptr_file) != v_num + 1 || read_array(&h_idx, idx_file) != e_num) {
+        cout << "cannot read " << ptr_file << " / " << idx_file << endl;
+        return 1;
+    }
+    default_random_engine engine;
+    engine.seed(123);
+    uniform_real_distribution<float> rd(0, 1);
+    vector<float> h_val(e_num, 1.0f), h_vin((size_t)v_num * last_dim), h_out((size_t)v_num * last_dim);
+    generate(h_vin.begin(), h_vin.end(), [&]() { return rd(engine); });
     float *val, *vin, *vout;
     hipMalloc(&val, e_num * sizeof(float));
-    hipMalloc(&vin, (size_t)v_num * last_dim * sizeof(float));
-    hipMalloc(&vout, (size_t)v_num * last_dim * sizeof(float));
+    hipMalloc(&vin, h_vin.size() * sizeof(float));
+    hipMalloc(&vout, h_out.size() * sizeof(float));
+    hipMemcpy(val, h_val.data(), e_num * sizeof(float), hipMemcpyHostToDevice);
+    hipMemcpy(vin, h_vin.data(), h_vin.size() * sizeof(float), hipMemcpyHostToDevice);
 
     SPMM_ACCEL accel(graph, ptr, idx, val, vin, vout, v_num, e_num, last_dim);
 
+    int rc = 0;
     for (int dim = first_dim; dim <= last_dim; dim += step) {
-        accel.do_test(false, dim);
+        cout << "CHECKING ..." << endl;
+        if (accel.do_test(false, dim) < 0) {
+            cout << "accel: " << accel.error() << endl;
+            return 1;
+        }
+        hipMemcpy(h_out.data(), vout, (size_t)v_num * dim * sizeof(float), hipMemcpyDeviceToHost);
+        vector<float> got(h_out.begin(), h_out.begin() + (size_t)v_num * dim), ref((size_t)v_num * dim, 0.0f);
+        for (int r = 0; r < v_num; r++)
+            for (int p = h_ptr[r]; p < h_ptr[r + 1]; p++)
+                for (int j = 0; j < dim; j++) ref[(size_t)r * dim + j] += h_val[p] * h_vin[(size_t)h_idx[p] * dim + j];
+        double err = mean_abs_diff(got, ref);
+        cout << "err mean = " << err << "  " << (err < 0.001 ? "validation pass!" : "validation fail!") << endl;
+        if (!(err < 0.001)) rc = 2;
+        cout << "TIMING ..." << endl;
         timestamp(t0);
         double t_accel = accel.do_test(true, dim);
         timestamp(t1);
-        cout << graph << " " << to_string(dim) << " accel " << t_accel * 1000000 << " (whole call "
-             << getDuration(t0, t1) << " s)" << endl;
+        cout << "0/0 " << graph << " " << to_string(dim) << " accel " << t_accel * 1000000 << endl;
+        cout << "whole call " << getDuration(t0, t1) << " s" << endl;
     }
-    vector<float> a(4, 0.f), b(4, 0.f);
-    cout << mean_abs_diff(a, b) << endl;
     hipFree(ptr); hipFree(idx); hipFree(val); hipFree(vin); hipFree(vout);
-    return 0;
+    delete[] h_ptr;
+    delete[] h_idx;
+    return rc;
 }
 
 int main(int argc, char *argv[])
 {
-    return argc > 1 ? run_graph(string(argv[1]), argc > 2) : 0;
+    if (argc < 3) {
+        cout << "usage: upstream_shaped_caller <graph> <dim> [natural]" << endl;
+        return 64;
+    }
+    first_dim = last_dim = atoi(argv[2]);
+    return run_graph(string(argv[1]), argc > 3);
 }

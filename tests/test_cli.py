@@ -136,3 +136,23 @@ def test_cli_natural_order_input(gpu, tmp_path):
     assert "loaded from saved state" not in third.stderr and "validation pass!" in third.stdout
     missing = subprocess.run(base + ["--natural", "nosuch", "40"], capture_output=True, text=True, timeout=120)
     assert missing.returncode != 0
+
+
+@pytest.mark.gpu
+def test_upstream_shaped_driver_runs_on_a_dataset_in_upstreams_layout(gpu, tmp_path):
+    """The driver of tests/cases (written like main.cu: data.h readers, `string` before its
+    using-directive, the nine-argument constructor, do_test(false/true, dim), util.h's clock)
+    reads ../graphs/<g>.* relative to its working directory (main.cu:10), as upstream does,
+    checks the operator against a host loop and prints upstream's timing line, for the
+    pre-sorted files and for the graph's own order."""
+    exe = EXE.parent / "upstream_shaped_caller"
+    assert exe.exists(), "upstream_shaped_caller was not built"
+    graphs, meta = write_graph(tmp_path, "mix", seed=16)
+    build = tmp_path / "build"
+    build.mkdir()
+    for extra in ([], ["natural"]):
+        r = subprocess.run([str(exe), "mix", "24"] + extra, cwd=build, capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, r.stdout + r.stderr
+        assert "validation pass!" in r.stdout and re.search(r"^0/0 mix 24 accel [0-9.eE+-]+$", r.stdout, re.M)
+    r = subprocess.run([str(exe), "nosuch", "24"], cwd=build, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 1 and "cannot read" in r.stdout

@@ -92,6 +92,39 @@ def test_after_a_loaded_state(gpu, tmp_path):
     b.close()
 
 
+def test_preprocessing_again_after_an_update_keeps_the_new_values(gpu, tmp_path):
+    """A handle that uploaded its CSR updates only its sorted copy; its copy of the caller's
+    order is brought back from there when the handle is preprocessed (or loads a state) again."""
+    g = graph(35)
+    N = 24
+    X = np.random.default_rng(15).uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    a = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    a.save_state(tmp_path / "g.accelstate")
+    v = new_values(g, 16)
+    dV = gpu.DeviceBuffer.from_numpy(v)
+    a.update_values_async(dV)
+    dV.close()                                            # the handle does not borrow it
+    want = a.matmul(X)
+    assert so.check(want, g.indptr, g.indices, v, X) <= TOL
+    a.preprocess(plan_unit=64)                            # other plan, same (new) values
+    assert so.check(a.matmul(X), g.indptr, g.indices, v, X) <= TOL
+    w = new_values(g, 17)
+    dW = gpu.DeviceBuffer.from_numpy(w)
+    a.update_values_async(dW)
+    a.update_values_async(dW)
+    a.load_state(tmp_path / "g.accelstate")               # the saved order, the newest values
+    got = a.matmul(X)
+    assert so.check(got, g.indptr, g.indices, w, X) <= TOL
+    b = gpu.AccelSpMM(g.indptr, g.indices, w, g.n_cols).preprocess()
+    assert np.array_equal(got.view(np.uint32), b.matmul(X).view(np.uint32))
+    a.update_values(v)                                    # a host array goes into the handle's copy directly
+    a.preprocess()
+    assert np.array_equal(a.matmul(X).view(np.uint32), want.view(np.uint32))
+    dW.close()
+    a.close()
+    b.close()
+
+
 def test_borrowed_device_csr(gpu):
     """A handle on the caller's device arrays: the same array rewritten in place, then another one."""
     g = graph(33)

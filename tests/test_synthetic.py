@@ -125,10 +125,20 @@ def test_bench_workload_cache_and_traffic_record(pkg, tmp_path):
         wl, n = key.rsplit("/N", 1)
         value, note = bench.recorded_traffic(wl, int(n))
         if e.get("source_sha16") == now:
-            assert value == e["traffic_bytes"] and note is None
+            assert value == e and note is None and value["traffic_bytes"] > 0 and 0 < value["l2_hit_rate"] < 1
         else:
             assert value is None and "taken with kernel sources" in note
     assert bench.recorded_traffic("cfg1", 7) == (None, "this workload was not profiled")
+    # the ceilings of the bench line: the probe's two rates come from the same committed file
+    rates = bench.probe_rates(64)
+    assert rates == entries["_probe_rates_GBps"]["N64"] and bench.probe_rates(16) == entries["_probe_rates_GBps"]["N16"]
+    assert bench.probe_rates(100) == rates and bench.probe_rates(20) == entries["_probe_rates_GBps"]["N32"]
+    alg, delivered = 2_256_466_672, 125_258_334 * 64 * 4          # the headline workload
+    all_hits, at_rate = bench.ceilings(alg, delivered, 0.3057, rates)
+    assert abs(all_hits - 0.234) < 5e-4 and abs(at_rate - 0.0815) < 5e-4
+    assert bench.ceilings(alg, delivered, 1.0, rates)[1] == pytest.approx(all_hits)
+    assert bench.ceilings(alg, delivered, None, rates) == (all_hits, None)
+    assert bench.ceilings(alg, delivered, 0.3, None) == (None, None)
 
 
 def test_export_in_upstreams_layout(pkg, tmp_path):
