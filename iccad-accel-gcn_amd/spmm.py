@@ -251,10 +251,10 @@ class AccelSpMM:
             dY.close()
 
     def time(self, X, Y, N: int, warmup: int = 4, iters: int = 20, stream=None, split: bool = True):
-        """HIP-event timings in ms: (total per run, gather kernel only).  With
-        ``split=False`` no event is recorded between the two kernels of a run (the
-        second array is then all zeros); use that for launches of a few microseconds,
-        where the extra event is a visible part of the total."""
+        """HIP-event timings in ms: (total per run, gather kernel only).  The total comes
+        from two events recorded around each run, the kernel's time from two events bound to
+        its own start and end (nothing is put between the kernels of a run).  With
+        ``split=False`` the kernel's events are left out (the second array is then all zeros)."""
         tot = np.zeros(iters, dtype=np.float32)
         main = np.zeros(iters, dtype=np.float32)
         x, y, _ = self._operands(X, Y, N)

@@ -35,7 +35,8 @@ typedef enum accel_status {
     ACCEL_ERR_ALLOC = -3,  /* host or device allocation failed */
     ACCEL_ERR_HIP = -4,    /* HIP runtime error (includes "no GPU") */
     ACCEL_ERR_META = -5,   /* supplied .block4 metadata does not describe this CSR */
-    ACCEL_ERR_STATE = -6,  /* call order violated (run before preprocess, ...) */
+    ACCEL_ERR_STATE = -6,  /* call order violated (run before preprocess, ...), another GPU current than the
+                              handle's, or a call that would have to allocate while its stream is capturing */
     ACCEL_ERR_IO = -7      /* file missing / truncated */
 } accel_status;
 
