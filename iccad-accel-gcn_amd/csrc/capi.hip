@@ -55,7 +55,8 @@ void release_products(accel_handle *h)
         sl = accel_handle::StreamSlot();
     }
     h->writer_done = nullptr; h->writer = nullptr; h->writer_pending = false;
-    h->partial_slot = -1; h->next_victim = 0; h->track_runs = false;
+    h->partial_slot = -1; h->next_victim = 0;
+    h->has_home = false; h->home = nullptr; h->multi_stream = false;
     h->perm = nullptr; h->s_indptr = nullptr; h->s_idx = nullptr; h->s_val = nullptr;
     h->work = nullptr; h->long_slot = nullptr; h->row_done = nullptr; h->block4 = nullptr; h->partial = nullptr;
     h->n_units = h->n_long_units = 0;
@@ -149,15 +150,16 @@ static int check_run(accel_handle *h, const float *X, float *Y, int32_t N, const
 // ---------------------------------------------------------------------------
 // Stream order of a handle's mutable device memory.  Runs read the sorted values and, when
 // the matrix has split rows, write and then read the partial-sum buffer; a value update
-// rewrites the sorted values.  Work queued on one stream is ordered by the stream.  Across
-// streams the handle orders it itself, on the device, without making the host wait: a
-// tracked run binds an event to its last kernel (no extra packet in the queue), kept in the
-// slot of its stream, and whatever has to come after that run on another stream waits for
-// the event.  Runs are tracked when the matrix has split rows (the shared buffer) and, from
-// the first value update on, always.  A stream is never touched after the call that used it
-// has returned, so the caller may destroy it at any time.  A stream that is capturing is
-// left alone (an event of work outside a capture cannot be waited for inside one): the
-// caller orders a graph against other uses of the handle.
+// rewrites the sorted values.  Work queued on one stream is ordered by the stream, and as
+// long as a handle is used on one stream only nothing else happens (an event per run costs
+// the run some 2 us on the device, a fifth of a launch-bound matrix's run).  The first use on
+// a second stream waits for the device once; from then on the handle orders its uses itself,
+// on the device, without making the host wait: a run binds an event to its last kernel, kept
+// in the slot of its stream, and whatever has to come after that run on another stream waits
+// for the event.  A stream is never touched after the call that used it has returned, so the
+// caller may destroy it at any time.  A stream that is capturing is left alone (an event of
+// work outside a capture cannot be waited for inside one, and the device cannot be waited
+// for): the caller orders a graph against other uses of the handle.
 // ---------------------------------------------------------------------------
 bool stream_is_capturing(hipStream_t s)
 {
@@ -169,12 +171,36 @@ bool stream_is_capturing(hipStream_t s)
     return cap != hipStreamCaptureStatusNone;
 }
 
+// Whether a call on s has to find out if s is capturing: only when it would do something a
+// capture does not allow.
+bool needs_capture_status(const accel_handle *h, hipStream_t s)
+{
+    return h->multi_stream || (h->has_home && s != h->home);
+}
+
+// One stream so far, or the switch to tracking when a second one turns up.  *single: the
+// handle still lives on one stream.
+static int single_stream(accel_handle *h, hipStream_t s, bool *single)
+{
+    *single = false;
+    if (h->multi_stream) return ACCEL_OK;
+    if (!h->has_home) { h->home = s; h->has_home = true; }
+    if (s == h->home) { *single = true; return ACCEL_OK; }
+    ACCEL_HIP(hipDeviceSynchronize());      // once per handle: what the first stream holds left no events
+    h->multi_stream = true;
+    h->writer_pending = false;
+    return ACCEL_OK;
+}
+
 // Before a run is queued on s.  *run_done receives the event to bind to the run's last kernel
 // (null: this run is not tracked).
 int order_run(accel_handle *h, hipStream_t s, bool uses_partial, bool capturing, hipEvent_t *run_done)
 {
     *run_done = nullptr;
     if (capturing) return ACCEL_OK;
+    bool single = false;
+    if (int rc = single_stream(h, s, &single)) return rc;
+    if (single) return ACCEL_OK;
     if (h->writer_pending && s != h->writer) {
         if (hipEventQuery(h->writer_done) == hipSuccess) {
             h->writer_pending = false;
@@ -183,7 +209,6 @@ int order_run(accel_handle *h, hipStream_t s, bool uses_partial, bool capturing,
             ACCEL_HIP(hipStreamWaitEvent(s, h->writer_done, 0));
         }
     }
-    if (!uses_partial && !h->track_runs) return ACCEL_OK;
     int mine = -1;
     for (int i = 0; i < accel_handle::kMaxStreams; i++)
         if (h->slot[i].done && h->slot[i].stream == s) mine = i;
@@ -216,11 +241,9 @@ int order_run(accel_handle *h, hipStream_t s, bool uses_partial, bool capturing,
 int order_update(accel_handle *h, hipStream_t s, bool capturing)
 {
     if (capturing) return ACCEL_OK;
-    if (!h->track_runs) {
-        // the first update of this handle: its runs so far left no events behind
-        ACCEL_HIP(hipDeviceSynchronize());
-        h->track_runs = true;
-    }
+    bool single = false;
+    if (int rc = single_stream(h, s, &single)) return rc;
+    if (single) return ACCEL_OK;
     for (auto &sl : h->slot)
         if (sl.live && sl.stream != s) ACCEL_HIP(hipStreamWaitEvent(s, sl.done, 0));
     if (h->writer_pending && h->writer != s) ACCEL_HIP(hipStreamWaitEvent(s, h->writer_done, 0));
@@ -230,7 +253,7 @@ int order_update(accel_handle *h, hipStream_t s, bool capturing)
 // Behind a value update queued on s.
 int note_update(accel_handle *h, hipStream_t s, bool capturing)
 {
-    if (capturing) return ACCEL_OK;
+    if (capturing || !h->multi_stream) return ACCEL_OK;
     if (!h->writer_done) ACCEL_HIP(hipEventCreateWithFlags(&h->writer_done, hipEventDisableTiming));
     ACCEL_HIP(hipEventRecord(h->writer_done, s));
     h->writer = s;

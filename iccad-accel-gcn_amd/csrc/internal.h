@@ -131,9 +131,14 @@ struct accel_handle {
     bool val_stale = false;
     // Which streams use the handle's mutable device memory (see order_run / order_update in
     // capi.hip).  Runs read the sorted values and, with split rows, write and read `partial`;
-    // a value update rewrites the sorted values.  A tracked run leaves an event, bound to its
-    // last kernel, in the slot of its stream; nothing is ever asked of a stream after the call
-    // that used it has returned (the caller may have destroyed it).
+    // a value update rewrites the sorted values.  As long as all of that happens on one stream
+    // (`home`), the stream orders it and nothing is tracked.  The first use on a second stream
+    // waits for the device once and switches the handle to tracking: from then on a run leaves
+    // an event, bound to its last kernel, in the slot of its stream.  Nothing is ever asked of
+    // a stream after the call that used it has returned (the caller may have destroyed it).
+    hipStream_t home = nullptr;              // the one stream the handle has been used on so far
+    bool has_home = false;
+    bool multi_stream = false;               // a second stream has turned up: runs are tracked
     static constexpr int kMaxStreams = 4;
     struct StreamSlot {
         hipStream_t stream = nullptr;
@@ -142,7 +147,6 @@ struct accel_handle {
     } slot[kMaxStreams];
     int next_victim = 0;                     // slot reused when a fifth stream turns up
     int partial_slot = -1;                   // slot of the last run that used `partial`
-    bool track_runs = false;                 // the values have been updated once: every run is tracked
     hipStream_t writer = nullptr;            // stream of the last value update
     bool writer_pending = false;             // ... which may still be running
     hipEvent_t writer_done = nullptr;        // recorded behind it
@@ -161,6 +165,7 @@ int restore_own_values(accel_handle *h, hipStream_t s);
 // capi.hip
 void release_products(accel_handle *h);
 bool stream_is_capturing(hipStream_t s);
+bool needs_capture_status(const accel_handle *h, hipStream_t s);
 int order_run(accel_handle *h, hipStream_t s, bool uses_partial, bool capturing, hipEvent_t *run_done);
 int order_update(accel_handle *h, hipStream_t s, bool capturing);
 int note_update(accel_handle *h, hipStream_t s, bool capturing);

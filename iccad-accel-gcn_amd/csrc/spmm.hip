@@ -797,9 +797,10 @@ int spmm_launch(accel_handle *h, const float *X, float *Y, int N, hipStream_t st
     // run needs more than it holds), or this GPU's static array, which is never allocated
     float *partial = h->partial;
     const bool uses_handle_partial = !static_partial && h->n_long_units > 0;
-    // the capture status is only needed where something depends on it
-    const bool capturing =
-        (uses_handle_partial || h->writer_pending || h->track_runs) && stream_is_capturing(stream);
+    // the capture status is only asked for where something depends on it: a buffer that would
+    // have to grow, or a stream the handle would have to order against another
+    const bool must_grow = uses_handle_partial && h->partial_floats < (size_t)h->n_long_units * (size_t)ld;
+    const bool capturing = (must_grow || needs_capture_status(h, stream)) && stream_is_capturing(stream);
     if (static_partial) {
         partial = nullptr;
         const size_t need = (size_t)h->n_long_units * (size_t)ld;

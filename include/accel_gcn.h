@@ -166,10 +166,11 @@ int accel_load_state(accel_handle *h, const char *path);
  *
  * accel_update_values_async: val_dev = nnz floats on the device in the order of the CSR
  * given to accel_create; the kernel is queued on `stream` (a hipStream_t, NULL = default
- * stream) and the call returns without waiting.  The handle orders it on the device
- * behind its own runs that are still in flight on other streams, and later runs on other
- * streams behind it, so "update, then run" needs no host synchronisation whatever the
- * streams are.  It can be captured into a HIP graph together with the runs that follow
+ * stream) and the call returns without waiting.  On the stream the handle's runs use it
+ * is ordered by that stream.  On another stream the handle orders it on the device behind
+ * its runs that are still in flight, and later runs on other streams behind it (see
+ * accel_run: the first call on a second stream waits for the device once), so "update,
+ * then run" needs no host synchronisation whatever the streams are.  It can be captured into a HIP graph together with the runs that follow
  * (after one update outside the capture has built the map; a capturing stream is only
  * ordered against itself).  A handle that borrows device arrays borrows val_dev from now
  * on (it may be the same array, rewritten in place); a handle that uploaded its CSR keeps
@@ -280,11 +281,12 @@ int accel_get_plan(const accel_handle *h, int32_t *out, int64_t cap_units, int64
  * except while `stream` is capturing: the runtime answers no such query during a capture),
  * and a call with another GPU current than the one the handle was created on with
  * ACCEL_ERR_STATE.  The partial-sum buffer of a matrix with split rows is shared by all
- * runs of the handle: a run on another stream than the previous one is made to wait, on
- * the device, for what that stream held at the time of the call (no error, no host
- * wait; runs on one stream are ordered anyway; distinct handles are independent).  A
- * stream that is capturing is not ordered against other streams: the caller orders a
- * graph against other uses of the handle. */
+ * runs of the handle.  A handle used on one stream needs nothing beyond the stream's own
+ * order.  The first call on a second stream waits for the device once; from then on every
+ * run of the handle carries an event and a run on another stream than the previous one is
+ * made to wait for that one on the device (no error, no host wait; distinct handles are
+ * independent).  A stream that is capturing is not ordered against other streams: the
+ * caller orders a graph against other uses of the handle. */
 int accel_run(accel_handle *h, const float *X, float *Y, int32_t N, void *stream);
 
 /* run with the rest of a GCN layer fused into the store: Y = act(A X + bias).
