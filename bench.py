@@ -379,6 +379,9 @@ def main():
             op.run_strided(sX, sY, N, a.ld)
         op.synchronize()
         strided = {"ld": a.ld, "ms_per_step": round((time.perf_counter() - t1) / a.steps * 1e3, 5)}
+        s_tot, s_main = op.time_ex(sX, sY, N, ld=a.ld, warmup=0, iters=a.steps)
+        strided["kernel_ms_avg"] = round(float(np.mean(s_main)), 5)
+        strided["all_kernels_ms_avg"] = round(float(np.mean(s_tot)), 5)
         sX.close()
         sY.close()
 

@@ -942,15 +942,14 @@ int accel_run_epilogue(accel_handle *h, const float *X, float *Y, int32_t N, con
                        (flags & ACCEL_EPILOGUE_RELU) ? 1 : 0);
 }
 
-int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup, int iters,
-               float *ms_total, float *ms_main, void *stream)
+// The timing protocol on any form of run: a->stream carries the launches.
+static int time_runs(accel_handle *h, const accel_run_args *a, int32_t ld, int warmup, int iters, float *ms_total,
+                     float *ms_main)
 {
-    clear_error();
-    if (warmup < 0 || iters < 0) { set_error("accel_time: bad warmup/iters"); return ACCEL_ERR_ARG; }
-    if (int rc = check_run(h, X, Y, N, nullptr, "accel_time", static_cast<hipStream_t>(stream))) return rc;
-    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipStream_t s = static_cast<hipStream_t>(a->stream);
+    const int relu = (a->flags & ACCEL_EPILOGUE_RELU) ? 1 : 0;
     for (int i = 0; i < warmup; i++)
-        if (int rc = spmm_launch(h, X, Y, N, s)) return rc;
+        if (int rc = spmm_launch(h, a->X, a->Y, a->N, s, nullptr, nullptr, a->bias, relu, false, ld)) return rc;
     ACCEL_HIP(hipStreamSynchronize(s));
     if (iters == 0) return ACCEL_OK;
     // All launches are queued back to back; the events are read after one final wait.  Per
@@ -963,7 +962,8 @@ int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup,
     for (int i = 0; i < iters && !rc; i++) {
         hipError_t e = hipEventRecord(ev[4 * i], s);
         if (e == hipSuccess)
-            rc = spmm_launch(h, X, Y, N, s, ms_main ? ev[4 * i + 1] : nullptr, ms_main ? ev[4 * i + 2] : nullptr);
+            rc = spmm_launch(h, a->X, a->Y, a->N, s, ms_main ? ev[4 * i + 1] : nullptr,
+                             ms_main ? ev[4 * i + 2] : nullptr, a->bias, relu, false, ld);
         if (!rc && e == hipSuccess) e = hipEventRecord(ev[4 * i + 3], s);
         if (!rc && e != hipSuccess) { set_error("hipEventRecord: %s", hipGetErrorString(e)); rc = ACCEL_ERR_HIP; }
     }
@@ -981,6 +981,29 @@ int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup,
     for (auto e : ev)
         if (e) (void)hipEventDestroy(e);
     return rc;
+}
+
+int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup, int iters,
+               float *ms_total, float *ms_main, void *stream)
+{
+    clear_error();
+    if (warmup < 0 || iters < 0) { set_error("accel_time: bad warmup/iters"); return ACCEL_ERR_ARG; }
+    if (int rc = check_run(h, X, Y, N, nullptr, "accel_time", static_cast<hipStream_t>(stream))) return rc;
+    const accel_run_args a{X, Y, N, 0, nullptr, 0, stream};
+    return time_runs(h, &a, N, warmup, iters, ms_total, ms_main);
+}
+
+int accel_time_ex(accel_handle *h, const accel_run_args *a, int warmup, int iters, float *ms_total,
+                  float *ms_main)
+{
+    clear_error();
+    if (!a) { set_error("accel_time_ex: null arguments"); return ACCEL_ERR_ARG; }
+    if (warmup < 0 || iters < 0) { set_error("accel_time_ex: bad warmup/iters"); return ACCEL_ERR_ARG; }
+    const int32_t ld = a->ld == 0 ? a->N : a->ld;
+    if (ld < a->N) { set_error("accel_time_ex: the row stride (%d) must be 0 or at least N (%d)", a->ld, a->N); return ACCEL_ERR_ARG; }
+    if (a->flags & ~ACCEL_EPILOGUE_RELU) { set_error("accel_time_ex: unknown flags %d", a->flags); return ACCEL_ERR_ARG; }
+    if (int rc = check_run(h, a->X, a->Y, a->N, a->bias, "accel_time_ex", static_cast<hipStream_t>(a->stream), ld)) return rc;
+    return time_runs(h, a, ld, warmup, iters, ms_total, ms_main);
 }
 
 }  // extern "C"

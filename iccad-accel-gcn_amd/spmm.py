@@ -262,6 +262,27 @@ class AccelSpMM:
                                ptr(tot, C.c_float), ptr(main, C.c_float) if split else None, ptr(stream)))
         return tot, main
 
+    def time_ex(self, X, Y, N: int, ld: int = 0, bias=None, relu=False, warmup: int = 4, iters: int = 20,
+                stream=None, split: bool = True):
+        """``time`` on a run with every option (see accel_time_ex): rows ``ld`` floats apart
+        (0: packed), Y = act(A X + bias)."""
+        N, ld = int(N), int(ld)
+        step = ld or N
+        if N <= 0 or step < N:
+            raise AccelError(_lib.ERR_ARG, f"need 0 < N <= ld (or ld = 0), got N={N}, ld={ld}")
+        a = _lib.RunArgs()
+        x = _lib.dev_ptr(X, ((self.n_cols - 1) * step + N) * 4 if self.n_cols else 0, "X")
+        y = _lib.dev_ptr(Y, ((self.n_rows - 1) * step + N) * 4 if self.n_rows else 0, "Y")
+        b = _lib.dev_ptr(bias, N * 4, "bias")
+        s = ptr(stream)
+        a.X, a.Y, a.N, a.ld = x.value if x else None, y.value if y else None, N, ld
+        a.bias, a.flags, a.stream = b.value if b else None, _lib.EPILOGUE_RELU if relu else 0, s.value if s else None
+        tot = np.zeros(iters, dtype=np.float32)
+        main = np.zeros(iters, dtype=np.float32)
+        check(lib().accel_time_ex(self._h, C.byref(a), warmup, iters, ptr(tot, C.c_float),
+                                  ptr(main, C.c_float) if split else None))
+        return tot, main
+
     def close(self) -> None:
         if self._h:
             lib().accel_destroy(self._h)

@@ -360,6 +360,11 @@ int accel_run_static(accel_handle *h, const float *X, float *Y, int32_t N, void 
 int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup, int iters,
                float *ms_total, float *ms_main, void *stream);
 
+/* The same protocol on a run with every option (rows `ld` apart, bias, ReLU): accel_time is
+ * this call with those fields at zero. */
+int accel_time_ex(accel_handle *h, const accel_run_args *args, int warmup, int iters, float *ms_total,
+                  float *ms_main);
+
 int accel_destroy(accel_handle *h);
 
 #ifdef __cplusplus

@@ -343,6 +343,34 @@ def test_timing_entry_point(gpu, mixed):
     dY.close()
 
 
+def test_timing_entry_point_with_every_option(gpu, mixed):
+    """accel_time_ex: the same protocol on rows with a stride, bias and ReLU; the output it
+    leaves is the product."""
+    g, op = mixed
+    N, ld = 50, 64
+    rng = np.random.default_rng(5)
+    X = rng.uniform(-1, 1, (g.n_cols, N)).astype(np.float32)
+    bias = rng.uniform(-1, 1, N).astype(np.float32)
+    Xp = np.zeros((g.n_cols, ld), np.float32); Xp[:, :N] = X
+    dX, dB = gpu.DeviceBuffer.from_numpy(Xp), gpu.DeviceBuffer.from_numpy(bias)
+    dY = gpu.DeviceBuffer(g.n_rows * ld * 4)
+    dY.fill_u32(0x7FC00000)
+    tot, main = op.time_ex(dX, dY, N, ld=ld, bias=dB, relu=True, warmup=1, iters=4)
+    assert tot.shape == (4,) and np.all(tot > 0) and np.all(main > 0) and np.all(main <= tot * 1.001)
+    Y = dY.to_numpy(np.float32, (g.n_rows, ld))
+    R, S = so.spmm_fp64(g.indptr, g.indices, g.values, X)
+    want = np.maximum(R + bias.astype(np.float64), 0.0)
+    assert np.max(np.abs(Y[:, :N] - want) / np.maximum(S + np.abs(bias), 1e-30)) <= TOL
+    assert np.isnan(Y[:, N:]).all()
+    L = gpu._lib
+    a = L.RunArgs()
+    a.X, a.Y, a.N, a.ld = dX.address, dY.address, N, N - 1
+    assert L.lib().accel_time_ex(op._h, a, 1, 1, None, None) == L.ERR_ARG      # stride below N
+    assert L.lib().accel_time_ex(op._h, None, 1, 1, None, None) == L.ERR_ARG
+    for b in (dX, dB, dY):
+        b.close()
+
+
 def test_medium_power_law_graph(gpu):
     """A 300k-row, ~15M-edge graph generated like cfg4 (gamma 2.1)."""
     g = gpu.synthetic.cfg4(n=300_000, n_edges=15_000_000, max_degree=17_000)
