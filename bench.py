@@ -200,6 +200,52 @@ def neighbor_partition_baseline(pkg, g, dX, N, iters=10):
     return out, Yn
 
 
+def gcn_layer_timing(pkg, op, g, N, K, steps):
+    """Z = F W (accel_dense_xw) alone, then the layer Y = relu(A (F W) + b): both on the host
+    clock over `steps` launches queued back to back, after 10 warm-ups; a sample of rows of Z
+    is checked against an fp64 product."""
+    rng = np.random.default_rng(5)
+    rows = g.n_cols
+    F = rng.uniform(-1, 1, (rows, K)).astype(np.float32)
+    W = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+    dF, dW, dZ = pkg.DeviceBuffer.from_numpy(F), pkg.DeviceBuffer.from_numpy(W), pkg.DeviceBuffer(rows * N * 4)
+    dB = pkg.DeviceBuffer.from_numpy(rng.standard_normal(N).astype(np.float32))
+    dY = pkg.DeviceBuffer(g.n_rows * N * 4)            # the layer's own output: the timed run's Y stays as it is
+
+    def timed(fn):
+        for _ in range(10):
+            fn()
+        op.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        op.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    dense_ms = timed(lambda: pkg.dense_xw(dF, dW, dZ, rows, K, N))
+    Z = dZ.to_numpy(np.float32, (rows, N))
+    idx = np.unique(np.concatenate([np.arange(min(rows, 2048)), rng.integers(0, rows, 4096), np.arange(max(0, rows - 2048), rows)]))
+    R = F[idx].astype(np.float64) @ W.astype(np.float64)
+    S = np.abs(F[idx].astype(np.float64)) @ np.abs(W.astype(np.float64))
+    err = float(np.max(np.abs(Z[idx] - R) / np.maximum(S, np.finfo(np.float32).tiny)))
+
+    def one_layer():
+        pkg.dense_xw(dF, dW, dZ, rows, K, N)
+        op.run_epilogue(dZ, dY, N, bias=dB, relu=True)
+    layer_ms = timed(one_layer)
+    dense_bytes = rows * K * 4 + rows * N * 4 + K * N * 4
+    out = {"K": K, "dense_ms": round(dense_ms, 5), "layer_ms": round(layer_ms, 5),
+           "dense_TFLOPs": round(2.0 * rows * K * N / (dense_ms * 1e-3) / 1e12, 2),
+           "dense_frac_of_fp32_matrix_peak": round(2.0 * rows * K * N / (dense_ms * 1e-3) / 1e12 / 157.3, 4),
+           "dense_algorithmic_bytes": dense_bytes,
+           "dense_GBps": round(dense_bytes / (dense_ms * 1e-3) / 1e9, 1),
+           "dense_frac_of_hbm_peak": round(dense_bytes / (dense_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+           "dense_scaled_error": err, "dense_rows_checked": int(idx.size), "dense_ok": bool(err <= 1e-5)}
+    for b in (dF, dW, dZ, dB, dY):
+        b.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -237,6 +283,10 @@ def main():
     ap.add_argument("--ld", type=int, default=0,
                     help="also time accel_run_strided with rows of X and Y this many floats apart (>= N), "
                          "on the host clock; reported as config.strided")
+    ap.add_argument("--dense-k", type=int, default=0, metavar="K",
+                    help="also time the dense product of a GCN layer, Z = F W with F cols x K and W K x N "
+                         "(accel_dense_xw), alone and in front of the sparse product with bias and ReLU in its "
+                         "store; reported as config.gcn_layer")
     ap.add_argument("--cache-dir", default="/tmp/accelgcn_bench_cache",
                     help="where generated workloads are kept between runs ('' = do not keep them)")
     a = ap.parse_args()
@@ -385,6 +435,8 @@ def main():
         sX.close()
         sY.close()
 
+    layer = gcn_layer_timing(pkg, op, g, N, a.dense_k, a.steps) if a.dense_k else None
+
     flops = 2.0 * g.nnz * N
     alg_bytes = g.nnz * 8 + g.n_cols * N * 4 + g.n_rows * N * 4
     main_avg_ms = float(np.mean(main_ms))
@@ -444,6 +496,8 @@ def main():
         result["roofline"]["traffic_stale"] = traffic_note + " (traffic, l2_hit_rate and the ceiling at the measured hit rate are null for that reason)"
     if strided:
         result["config"]["strided"] = strided
+    if layer:
+        result["config"]["gcn_layer"] = layer
 
     if a.compare_rocsparse:
         rs, Yr = rocsparse_baseline(pkg, op, g, dX, N)

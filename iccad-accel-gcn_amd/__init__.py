@@ -6,7 +6,8 @@ The directory name is not a Python identifier; load it with
 """
 from ._lib import AccelError, DeviceBuffer, device_count, lib  # noqa: F401
 from .spmm import AccelSpMM, SpmmAccel  # noqa: F401
+from .dense import GcnLayer, dense_xw, dense_xw_numpy  # noqa: F401
 from . import block_level_partition, synthetic  # noqa: F401
 
-__all__ = ["AccelError", "AccelSpMM", "DeviceBuffer", "SpmmAccel", "block_level_partition",
-           "device_count", "lib", "synthetic"]
+__all__ = ["AccelError", "AccelSpMM", "DeviceBuffer", "GcnLayer", "SpmmAccel", "block_level_partition",
+           "dense_xw", "dense_xw_numpy", "device_count", "lib", "synthetic"]

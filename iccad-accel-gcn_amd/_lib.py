@@ -99,6 +99,7 @@ SIGNATURES = {
     "accel_run_epilogue": (C.c_int, [vp, vp, vp, C.c_int32, vp, C.c_int, vp]),
     "accel_time": (C.c_int, [vp, vp, vp, C.c_int32, C.c_int, C.c_int, f32p, f32p, vp]),
     "accel_time_ex": (C.c_int, [vp, C.POINTER(RunArgs), C.c_int, C.c_int, f32p, f32p]),
+    "accel_dense_xw": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp]),
     "accel_destroy": (C.c_int, [vp]),
 }
 

@@ -17,7 +17,7 @@ CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB = LIB_DIR / "libaccelgcn.so"
 BIN_DIR = PKG / "bin"
-SOURCES = ["capi.hip", "preprocess.hip", "spmm.hip", "state.hip", "spmm_accel.cpp"]
+SOURCES = ["capi.hip", "preprocess.hip", "spmm.hip", "state.hip", "dense.hip", "spmm_accel.cpp"]
 ARCH = "gfx950"
 
 

@@ -26,6 +26,8 @@ void clear_error() { g_error.clear(); }
 int partition_only_device(const int32_t *indptr_dev, int64_t rows, int64_t nnz,
                           int32_t **block4_dev, int64_t *n_blocks);
 bool stream_is_capturing(hipStream_t s);
+int dense_xw_launch(const float *X, const float *W, float *Z, int64_t rows, int K, int N, int64_t ldx, int64_t ldz,
+                    hipStream_t stream);      // dense.hip
 
 void release_products(accel_handle *h)
 {
@@ -1004,6 +1006,42 @@ int accel_time_ex(accel_handle *h, const accel_run_args *a, int warmup, int iter
     if (a->flags & ~ACCEL_EPILOGUE_RELU) { set_error("accel_time_ex: unknown flags %d", a->flags); return ACCEL_ERR_ARG; }
     if (int rc = check_run(h, a->X, a->Y, a->N, a->bias, "accel_time_ex", static_cast<hipStream_t>(a->stream), ld)) return rc;
     return time_runs(h, a, ld, warmup, iters, ms_total, ms_main);
+}
+
+int accel_dense_xw(const float *X, const float *W, float *Z, int64_t rows, int32_t K, int32_t N, int32_t ldx,
+                   int32_t ldz, void *stream)
+{
+    clear_error();
+    const char *fn = "accel_dense_xw";
+    if (int rc = need_gpu()) return rc;
+    if (rows < 0 || K <= 0 || N <= 0) {
+        set_error("%s: bad shape (%lld rows, K = %d, N = %d)", fn, (long long)rows, K, N);
+        return ACCEL_ERR_ARG;
+    }
+    if (ldx == 0) ldx = K;
+    if (ldz == 0) ldz = N;
+    if (ldx < K || ldz < N) {
+        set_error("%s: row strides (%d, %d) must be 0 or at least K (%d) and N (%d)", fn, ldx, ldz, K, N);
+        return ACCEL_ERR_ARG;
+    }
+    if (rows == 0) return ACCEL_OK;
+    if (!X || !W || !Z) { set_error("%s: null operand", fn); return ACCEL_ERR_ARG; }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (!stream_is_capturing(s)) {              // see check_operand
+        const size_t x_bytes = ((size_t)(rows - 1) * (size_t)ldx + (size_t)K) * sizeof(float);
+        const size_t z_bytes = ((size_t)(rows - 1) * (size_t)ldz + (size_t)N) * sizeof(float);
+        if (int rc = check_operand(X, x_bytes, fn, "X")) return rc;
+        if (int rc = check_operand(W, (size_t)K * (size_t)N * sizeof(float), fn, "W")) return rc;
+        if (int rc = check_operand(Z, z_bytes, fn, "Z")) return rc;
+        const char *zb = reinterpret_cast<const char *>(Z), *xb = reinterpret_cast<const char *>(X),
+                   *wb = reinterpret_cast<const char *>(W);
+        if ((zb < xb + x_bytes && xb < zb + z_bytes) ||
+            (zb < wb + (size_t)K * N * sizeof(float) && wb < zb + z_bytes)) {
+            set_error("%s: Z overlaps an input", fn);
+            return ACCEL_ERR_ARG;
+        }
+    }
+    return dense_xw_launch(X, W, Z, rows, K, N, ldx, ldz, s);
 }
 
 }  // extern "C"

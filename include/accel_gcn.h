@@ -365,6 +365,19 @@ int accel_time(accel_handle *h, const float *X, float *Y, int32_t N, int warmup,
 int accel_time_ex(accel_handle *h, const accel_run_args *args, int warmup, int iters, float *ms_total,
                   float *ms_main);
 
+/* Z = X W in fp32: the dense product of a GCN layer, whose result is the dense operand of
+ * accel_run (layer: Y = act(A (X W) + bias) = accel_dense_xw, then accel_run_epilogue).  No
+ * counterpart upstream, whose operator takes the product as given (spmm_accel.cu:16-102 stops
+ * at A X).  X: rows x K floats, rows ldx floats apart (0 = K); W: K x N floats, packed
+ * row-major; Z: rows x N floats, rows ldz apart (0 = N; the columns N .. ldz-1 are not
+ * written); all three on the device, Z overlapping neither input.  Any rows >= 0, K >= 1,
+ * N >= 1; rows of X that start and end on 16-byte boundaries (X aligned, ldx and K multiples
+ * of 4) are read as 16-byte vectors.  Needs no handle; asynchronous on `stream`; allocates nothing.
+ * Computed on the fp32 matrix cores: sums of K products in fp32, whose order differs from a
+ * sequential loop (compare against a higher-precision product, as for accel_run). */
+int accel_dense_xw(const float *X, const float *W, float *Z, int64_t rows, int32_t K, int32_t N,
+                   int32_t ldx, int32_t ldz, void *stream);
+
 int accel_destroy(accel_handle *h);
 
 #ifdef __cplusplus

@@ -62,3 +62,20 @@ def upstream_mean_abs_error(Y, Yref):
 def check(Y, indptr, indices, values, X, tol=TOL):
     R, S = spmm_fp64(indptr, indices, values, X)
     return scaled_error(Y, R, S)
+
+
+# --- the dense product in front of the sparse one (Z = X W) -------------------------------
+# No reference counterpart (upstream's operator stops at A X, spmm_accel.cu:16-102): the
+# definition is the textbook matrix product, computed here by numpy in fp64.  Pinned by a
+# triple loop on small inputs, identity -> X, all-ones -> row sums, and a dropped-term
+# detector (tests/test_oracle_spmm.py).
+def dense_fp64(X, W):
+    """(R, S): X W in fp64 and |X| |W| in fp64 (the scale of the terms)."""
+    X64 = np.asarray(X, dtype=np.float64)
+    W64 = np.asarray(W, dtype=np.float64)
+    return X64 @ W64, np.abs(X64) @ np.abs(W64)
+
+
+def check_dense(Z, X, W):
+    R, S = dense_fp64(X, W)
+    return scaled_error(Z, R, S)

@@ -91,3 +91,23 @@ def test_threaded_fp64_oracle_is_the_same_routine_on_row_ranges():
     assert np.array_equal(R1, R2) and np.array_equal(S1, S2)
     R3, S3 = c_oracle.spmm_csr_f64(g.indptr[50:201], g.indices, g.values, X, threads=3)   # a slab of rows
     assert np.array_equal(R3, R1[50:200]) and np.array_equal(S3, S1[50:200])
+
+
+def test_dense_product_oracle():
+    rng = np.random.default_rng(5)
+    X = rng.standard_normal((9, 6)).astype(np.float32)
+    W = rng.standard_normal((6, 4)).astype(np.float32)
+    R, S = so.dense_fp64(X, W)
+    ref = np.zeros((9, 4)); ref_abs = np.zeros((9, 4))
+    for i in range(9):
+        for j in range(4):
+            for k in range(6):
+                ref[i, j] += float(X[i, k]) * float(W[k, j])
+                ref_abs[i, j] += abs(float(X[i, k])) * abs(float(W[k, j]))
+    assert np.allclose(R, ref, rtol=0, atol=1e-13) and np.allclose(S, ref_abs, rtol=0, atol=1e-13)
+    assert np.array_equal(so.dense_fp64(X, np.eye(6, dtype=np.float32))[0], X.astype(np.float64))
+    assert np.allclose(so.dense_fp64(X, np.ones((6, 3), np.float32))[0], X.astype(np.float64).sum(1)[:, None])
+    assert so.check_dense((X.astype(np.float64) @ W).astype(np.float32), X, W) <= so.TOL
+    Wt = W.copy(); Wt[2, 1] = 0.0                          # a dropped term is noticed
+    assert so.check_dense((X @ Wt).astype(np.float32), X, W) > 100 * so.TOL
+    assert so.check_dense((X[:, ::-1] @ W).astype(np.float32), X, W) > 100 * so.TOL      # a transposed index
