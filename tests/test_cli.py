@@ -156,3 +156,36 @@ def test_upstream_shaped_driver_runs_on_a_dataset_in_upstreams_layout(gpu, tmp_p
         assert "validation pass!" in r.stdout and re.search(r"^0/0 mix 24 accel [0-9.eE+-]+$", r.stdout, re.M)
     r = subprocess.run([str(exe), "nosuch", "24"], cwd=build, capture_output=True, text=True, timeout=120)
     assert r.returncode == 1 and "cannot read" in r.stdout
+
+
+@pytest.mark.gpu
+def test_bench_line_on_the_small_workload(gpu, tmp_path):
+    """bench.py end to end on the CPU-runnable workload, with every optional section: one JSON
+    line with the metric, the roofline and cpu_baseline objects, a passing parity check, the
+    strided run, both comparison baselines and the dense product of the layer."""
+    import json
+    import sys
+    r = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--workload", "cfg1", "--steps", "3", "--warmup", "2",
+                        "--ld", "64", "--dense-k", "48", "--compare-rocsparse", "--compare-neighbor-partition",
+                        "--cache-dir", str(tmp_path)], capture_output=True, text=True, timeout=600, cwd=str(ROOT))
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1, "exactly one line on stdout"
+    d = json.loads(lines[0])
+    assert d["metric"].startswith("SpMM GFLOP/s") and d["unit"] == "GFLOP/s" and d["n_gpus"] == 1
+    assert d["steps"] == 3 and d["warmup"] == 2 and d["dtype"] == "f32" and d["vs_baseline"] is None
+    assert d["value"] > 0 and d["ms_per_step"] > 0 and "cfg1" in d["config"]["workload"]
+    roof = d["roofline"]
+    assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and 0 < roof["frac"] < 1
+    assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
+    assert roof["algorithmic_bytes"] == d["config"]["nnz"] * 8 + 2 * d["config"]["rows"] * d["config"]["N"] * 4
+    assert d["cpu_baseline"]["kind"] == "port" and d["cpu_baseline"]["cores"] == 1 and d["cpu_baseline"]["value"] > 0
+    assert d["parity"]["ok"] and d["parity"]["rows_checked"] == d["config"]["rows"]
+    assert d["config"]["strided"]["ld"] == 64 and d["config"]["strided"]["kernel_ms_avg"] > 0
+    layer = d["config"]["gcn_layer"]
+    assert layer["K"] == 48 and layer["dense_ok"] and layer["layer_ms"] >= layer["dense_ms"] > 0
+    assert d["rocsparse"]["best_ms"] > 0 and d["neighbor_partition"]["ms"] > 0
+    # more than one GPU is refused with a message
+    r2 = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                        timeout=120, cwd=str(ROOT))
+    assert r2.returncode != 0 and "one GPU" in (r2.stdout + r2.stderr)
