@@ -11,6 +11,8 @@
 // per row) into registers two steps ahead and its 32 x (32 NT) block of W one step ahead,
 // while the matrix cores work on the steps before, then hands them over through LDS, where a
 // lane finds its row's 16 values of the step as four 16-byte reads.
+#include <atomic>
+
 #include "internal.h"
 
 namespace accel {
@@ -196,14 +198,25 @@ __global__ __launch_bounds__(kDenseThreads, NT == 4 ? 2 : 3) void dense_xw_kerne
 }
 
 // The grid: as many workgroups as the GPU holds at once (asked of the runtime for the kernel
-// that runs), or one per block of rows when there are fewer.
+// that runs, once per device and kernel), or one per block of rows when there are fewer.
+constexpr int kDenseDevices = 64;
+static std::atomic<int> g_resident[kDenseDevices][6];     // [device][kernel]: workgroups the device holds, 0 = not asked yet
+
 template <int NT, bool kVec>
 static int dense_launch(hipStream_t s, const float *X, const float *W, float *Z, int64_t rows, int K, int N, int64_t ldx,
-                        int64_t ldz, int64_t n_row_blocks, int n_col_tiles, int cus)
+                        int64_t ldz, int64_t n_row_blocks, int n_col_tiles)
 {
-    int per_cu = 0;
-    ACCEL_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, dense_xw_kernel<NT, kVec>, kDenseThreads, 0));
-    const int64_t resident = (int64_t)cus * (per_cu > 0 ? per_cu : 1);
+    constexpr int which = (NT == 1 ? 0 : NT == 2 ? 2 : 4) + (kVec ? 1 : 0);
+    int dev = 0;
+    ACCEL_HIP(hipGetDevice(&dev));
+    int resident = dev >= 0 && dev < kDenseDevices ? g_resident[dev][which].load(std::memory_order_relaxed) : 0;
+    if (resident == 0) {
+        int cus = 0, per_cu = 0;
+        ACCEL_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        ACCEL_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, dense_xw_kernel<NT, kVec>, kDenseThreads, 0));
+        resident = (cus > 0 ? cus : 256) * (per_cu > 0 ? per_cu : 1);
+        if (dev >= 0 && dev < kDenseDevices) g_resident[dev][which].store(resident, std::memory_order_relaxed);
+    }
     const unsigned grid = (unsigned)(n_row_blocks < resident ? n_row_blocks : resident);
     dense_xw_kernel<NT, kVec><<<grid, kDenseThreads, 0, s>>>(X, W, Z, rows, K, N, ldx, ldz, n_row_blocks, n_col_tiles);
     return ACCEL_OK;
@@ -218,16 +231,12 @@ int dense_xw_launch(const float *X, const float *W, float *Z, int64_t rows, int 
     const int nt = N <= 32 ? 1 : N <= 64 ? 2 : 4;
     const int n_col_tiles = (N + nt * 32 - 1) / (nt * 32);
     const int64_t n_row_blocks = (rows + kDenseBlockRows - 1) / kDenseBlockRows;
-    int dev = 0, cus = 0;
-    ACCEL_HIP(hipGetDevice(&dev));
-    ACCEL_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    if (cus <= 0) cus = 256;
     // 16-byte reads of X need every row to start on a 16-byte boundary and to end on one
     const bool vec = (reinterpret_cast<uintptr_t>(X) % 16 == 0) && (ldx % 4 == 0) && (K % 4 == 0);
     int rc;
-#define DENSE_CASE(NT_)                                                                                              \
-    rc = vec ? dense_launch<NT_, true>(stream, X, W, Z, rows, K, N, ldx, ldz, n_row_blocks, n_col_tiles, cus)       \
-             : dense_launch<NT_, false>(stream, X, W, Z, rows, K, N, ldx, ldz, n_row_blocks, n_col_tiles, cus)
+#define DENSE_CASE(NT_)                                                                                  \
+    rc = vec ? dense_launch<NT_, true>(stream, X, W, Z, rows, K, N, ldx, ldz, n_row_blocks, n_col_tiles)  \
+             : dense_launch<NT_, false>(stream, X, W, Z, rows, K, N, ldx, ldz, n_row_blocks, n_col_tiles)
     if (nt == 1) DENSE_CASE(1);
     else if (nt == 2) DENSE_CASE(2);
     else DENSE_CASE(4);
