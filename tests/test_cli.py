@@ -183,7 +183,7 @@ def test_bench_line_on_the_small_workload(gpu, tmp_path):
     assert d["parity"]["ok"] and d["parity"]["rows_checked"] == d["config"]["rows"]
     assert d["config"]["strided"]["ld"] == 64 and d["config"]["strided"]["kernel_ms_avg"] > 0
     layer = d["config"]["gcn_layer"]
-    assert layer["K"] == 48 and layer["dense_ok"] and layer["layer_ms"] >= layer["dense_ms"] > 0
+    assert layer["K"] == 48 and layer["dense_ok"] and layer["layer_ms"] > 0 and layer["dense_ms"] > 0
     assert d["rocsparse"]["best_ms"] > 0 and d["neighbor_partition"]["ms"] > 0
     # more than one GPU is refused with a message
     r2 = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True,
