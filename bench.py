@@ -200,7 +200,7 @@ def neighbor_partition_baseline(pkg, g, dX, N, iters=10):
     return out, Yn
 
 
-def gcn_layer_timing(pkg, op, g, N, K, steps):
+def gcn_layer_timing(pkg, op, g, N, K, steps, compare_rocblas=False):
     """Z = F W (accel_dense_xw) alone, then the layer Y = relu(A (F W) + b): both on the host
     clock over `steps` launches queued back to back; a sample of rows of Z is checked against
     an fp64 product.  The dense product alone is warmed up for 80 launches: a burst of
@@ -246,6 +246,23 @@ def gcn_layer_timing(pkg, op, g, N, K, steps):
            "dense_GBps": round(dense_bytes / (dense_ms * 1e-3) / 1e9, 1),
            "dense_frac_of_hbm_peak": round(dense_bytes / (dense_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
            "dense_scaled_error": err, "dense_rows_checked": int(idx.size), "dense_ok": bool(err <= 1e-5)}
+    if compare_rocblas:
+        # both sides the same way: the host clock over `steps` launches queued back to back, after 80 warm-ups
+        import ctypes as C
+        L = C.CDLL(os.path.join(os.path.dirname(str(pkg._lib.LIB_PATH)), "libaccelgcn_baselines.so"))
+        L.baseline_rocblas_last_error.restype = C.c_char_p
+        ms, queued = (C.c_float * steps)(), C.c_float(0)
+        rc = L.baseline_rocblas_sgemm(C.c_void_p(dF.address), C.c_void_p(dW.address), C.c_void_p(dZ.address),
+                                      C.c_int64(rows), C.c_int32(K), C.c_int32(N), 80, steps, ms, C.byref(queued))
+        if rc != 0:
+            out["rocblas"] = {"error": L.baseline_rocblas_last_error().decode()}
+        else:
+            Zr = dZ.to_numpy(np.float32, (rows, N))
+            theirs = float(queued.value)
+            out["rocblas"] = {"sgemm_ms": round(theirs, 5), "sgemm_ms_by_events_median": round(float(np.median(list(ms))), 5),
+                              "ours_ms": out["dense_ms"],
+                              "speedup": round(theirs / out["dense_ms"], 3),
+                              "max_abs_diff": float(np.max(np.abs(Zr[idx] - Z[idx])))}
     for b in (dF, dW, dZ, dB, dY):
         b.close()
     return out
@@ -292,6 +309,8 @@ def main():
                     help="also time the dense product of a GCN layer, Z = F W with F cols x K and W K x N "
                          "(accel_dense_xw), alone and in front of the sparse product with bias and ReLU in its "
                          "store; reported as config.gcn_layer")
+    ap.add_argument("--compare-rocblas", action="store_true",
+                    help="with --dense-k: also time rocBLAS SGEMM on the same dense operands (comparison only)")
     ap.add_argument("--cache-dir", default="/tmp/accelgcn_bench_cache",
                     help="where generated workloads are kept between runs ('' = do not keep them)")
     a = ap.parse_args()
@@ -440,7 +459,7 @@ def main():
         sX.close()
         sY.close()
 
-    layer = gcn_layer_timing(pkg, op, g, N, a.dense_k, a.steps) if a.dense_k else None
+    layer = gcn_layer_timing(pkg, op, g, N, a.dense_k, a.steps, a.compare_rocblas) if a.dense_k else None
 
     flops = 2.0 * g.nnz * N
     alg_bytes = g.nnz * 8 + g.n_cols * N * 4 + g.n_rows * N * 4

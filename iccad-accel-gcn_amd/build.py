@@ -70,13 +70,14 @@ def build(verbose: bool = False) -> Path:
 
 
 def build_baselines(verbose: bool = False) -> Path:
-    """lib/libaccelgcn_baselines.so: comparison baselines (rocSPARSE SpMM and a
-    neighbour-partition kernel) and the pure-gather measurement probe.  Kept in its own library: the product library does
+    """lib/libaccelgcn_baselines.so: comparison baselines (rocSPARSE SpMM, a
+    neighbour-partition kernel, rocBLAS SGEMM) and the pure-gather measurement probe.  Kept in its own library: the product library does
     not link any sparse library and holds no comparison code."""
     out = LIB_DIR / "libaccelgcn_baselines.so"
     cmd = [hipcc(), *compile_flags(), "-shared", str(PKG / "baselines" / "rocsparse_spmm.cpp"),
            str(PKG / "baselines" / "neighbor_partition_spmm.cpp"),
-           str(PKG / "baselines" / "gather_probe.cpp"), "-o", str(out), "-lrocsparse"]
+           str(PKG / "baselines" / "gather_probe.cpp"), str(PKG / "baselines" / "rocblas_gemm.cpp"),
+           "-o", str(out), "-lrocsparse", "-lrocblas"]
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

@@ -79,3 +79,20 @@ def test_gather_probe_runs(gpu, baselines):
         assert (stored.value > 0) == (stores != 0)
     assert baselines.baseline_gather_probe(C.c_int64(1000), C.c_int32(48), C.c_int32(8), C.c_int32(4), C.c_int32(0),
                                            C.c_int32(1), C.byref(ms), None, None) != 0      # N must be 16, 64 or 256
+
+
+def test_rocblas_baseline_computes_the_dense_product(gpu, baselines):
+    baselines.baseline_rocblas_last_error.restype = C.c_char_p
+    rng = np.random.default_rng(8)
+    rows, K, N = 1000, 48, 40
+    X = rng.uniform(-1, 1, (rows, K)).astype(np.float32)
+    W = rng.standard_normal((K, N)).astype(np.float32)
+    dX, dW, dZ = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer.from_numpy(W), gpu.DeviceBuffer(rows * N * 4)
+    ms, queued = (C.c_float * 2)(), C.c_float(0)
+    rc = baselines.baseline_rocblas_sgemm(C.c_void_p(dX.address), C.c_void_p(dW.address), C.c_void_p(dZ.address),
+                                          C.c_int64(rows), C.c_int32(K), C.c_int32(N), 1, 2, ms, C.byref(queued))
+    assert rc == 0, baselines.baseline_rocblas_last_error().decode()
+    assert so.check_dense(dZ.to_numpy(np.float32, (rows, N)), X, W) <= so.TOL
+    assert all(t > 0 for t in ms) and queued.value > 0
+    for b in (dX, dW, dZ):
+        b.close()
