@@ -115,6 +115,15 @@ static int check_operand(const void *p, size_t bytes, const char *fn, const char
     return ACCEL_OK;
 }
 
+// A CSR borrowed from the caller (ACCEL_PTR_DEVICE) must be device memory of the stated sizes.
+int check_borrowed_csr(const accel_handle *h, const char *fn)
+{
+    if (h->owns_input) return ACCEL_OK;
+    if (int rc = check_operand(h->indptr, sizeof(int32_t) * (size_t)(h->rows + 1), fn, "indptr")) return rc;
+    if (int rc = check_operand(h->idx, sizeof(int32_t) * (size_t)h->nnz, fn, "idx")) return rc;
+    return check_operand(h->val, sizeof(float) * (size_t)h->nnz, fn, "val");
+}
+
 // The handle's device memory belongs to the GPU it was created on; a launch with another GPU
 // current would hand that GPU addresses it cannot use.
 static int check_device(const accel_handle *h, const char *fn)
@@ -512,6 +521,8 @@ int accel_create(const int32_t *indptr, const int32_t *idx, const float *val, in
     if (flags == ACCEL_PTR_DEVICE) {
         h->indptr = indptr; h->idx = idx; h->val = val;
         h->owns_input = false;
+        // the kernels of accel_preprocess read these arrays: a host address would be a memory fault
+        if (int rc = check_borrowed_csr(h, "accel_create")) { delete h; return rc; }
     } else {
         void *a = nullptr, *b = nullptr, *c = nullptr;
         const size_t sa = sizeof(int32_t) * (size_t)(rows + 1);
@@ -647,6 +658,8 @@ int accel_preprocess(accel_handle *h)
 {
     clear_error();
     if (!h) { set_error("accel_preprocess: null handle"); return ACCEL_ERR_ARG; }
+    if (int rc = check_device(h, "accel_preprocess")) return rc;
+    if (int rc = check_borrowed_csr(h, "accel_preprocess")) return rc;     // still there, still large enough
     if (h->val_stale) {                     // value updates since: the handle's copy of the values first
         if (hipDeviceSynchronize() != hipSuccess) (void)hipGetLastError();
         if (int rc = restore_own_values(h, nullptr)) return rc;

@@ -23,6 +23,7 @@
 #include "internal.h"
 
 namespace accel {
+int check_borrowed_csr(const accel_handle *h, const char *fn);      // capi.hip
 namespace {
 
 constexpr char kMagic[8] = {'A', 'C', 'G', 'C', 'N', 'S', 'T', '2'};
@@ -135,6 +136,7 @@ int accel_load_state(accel_handle *h, const char *path)
 {
     clear_error();
     if (!h || !path) { set_error("accel_load_state: null argument"); return ACCEL_ERR_ARG; }
+    if (int rc = check_borrowed_csr(h, "accel_load_state")) return rc;
     const auto t0 = std::chrono::steady_clock::now();
     File in;
     in.f = fopen(path, "rb");

@@ -96,7 +96,10 @@ int accel_stream_sync(void *stream); /* NULL = default stream */
 /* ---- the operator ----------------------------------------------------------
  * init: replaces SPMM_BASE's constructor (spmm_base.h:9-20) for the CSR part:
  * stores (ACCEL_PTR_DEVICE) or uploads (ACCEL_PTR_HOST) the CSR.  The CSR may
- * be in any row order. */
+ * be in any row order.  Arrays passed as ACCEL_PTR_DEVICE are borrowed until
+ * accel_destroy and must be memory the GPU can read, of at least rows + 1, nnz and nnz
+ * elements: a host address or a smaller allocation is ACCEL_ERR_ARG here and again
+ * in accel_preprocess / accel_load_state, before any kernel reads them. */
 int accel_create(const int32_t *indptr, const int32_t *idx, const float *val, int64_t rows,
                  int64_t cols, int64_t nnz, int flags, accel_handle **out);
 

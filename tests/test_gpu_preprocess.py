@@ -152,6 +152,43 @@ def test_bad_csr_is_rejected(gpu):
         op.close()
 
 
+def test_borrowed_csr_must_be_device_memory(gpu):
+    """A CSR passed as device memory is read by kernels: host arrays, and device arrays
+    smaller than the stated sizes, are refused before anything is launched."""
+    import ctypes as C
+    lib, E = gpu.lib(), gpu._lib
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=2, n_long=2), seed=2)
+    host = [np.ascontiguousarray(a) for a in (g.indptr, g.indices, g.values)]
+    dev = [gpu.DeviceBuffer.from_numpy(a) for a in host]
+    h = C.c_void_p()
+
+    def create(ip, ix, v, rows=g.n_rows, nnz=g.nnz):
+        return lib.accel_create(C.c_void_p(ip), C.c_void_p(ix), C.c_void_p(v), rows, g.n_cols, nnz, E.PTR_DEVICE,
+                                C.byref(h))
+    addr = [d.address for d in dev]
+    for k in range(3):                                     # each array in turn as a host address
+        mixed = list(addr)
+        mixed[k] = host[k].ctypes.data
+        assert create(*mixed) == E.ERR_ARG and not h.value
+        assert "not memory the GPU can access" in E.last_error()
+    assert create(*addr, rows=g.n_rows + 1) == E.ERR_ARG   # indptr too small for one more row
+    assert create(*addr, nnz=g.nnz + 1) == E.ERR_ARG       # idx and val too small
+    assert "needs" in E.last_error()
+    assert create(*addr) == 0 and h.value
+    E.check(lib.accel_preprocess(h))
+    # the arrays are asked about again when the handle is preprocessed: freed since, refused
+    dev[1].close()
+    small = gpu.DeviceBuffer(16)
+    rc = lib.accel_preprocess(h)
+    assert rc in (0, E.ERR_ARG)                            # 0 only if the address is still mapped and large enough
+    if rc == E.ERR_ARG:
+        assert "idx" in E.last_error()
+    lib.accel_destroy(h)
+    small.close()
+    for d in (dev[0], dev[2]):
+        d.close()
+
+
 def test_stale_metadata_is_rejected(gpu):
     g = helpers.graph_from_degrees(np.sort(helpers.degree_mix(seed=1)), seed=1)
     op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
