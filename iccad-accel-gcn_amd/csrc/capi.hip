@@ -470,6 +470,8 @@ int accel_dev_fill_u32(void *dst, uint32_t value, size_t n_words, void *stream)
 {
     clear_error();
     if (n_words && !dst) { set_error("accel_dev_fill_u32: null argument"); return ACCEL_ERR_ARG; }
+    if (!stream_is_capturing(static_cast<hipStream_t>(stream)))          // see check_operand
+        if (int rc = check_operand(dst, n_words * 4, "accel_dev_fill_u32", "dst")) return rc;
     return fill_u32(dst, value, n_words, static_cast<hipStream_t>(stream));
 }
 
@@ -477,6 +479,10 @@ int accel_dev_copy_u32(void *dst_dev, const void *src_dev, size_t n_words, void 
 {
     clear_error();
     if (n_words && (!dst_dev || !src_dev)) { set_error("accel_dev_copy_u32: null argument"); return ACCEL_ERR_ARG; }
+    if (!stream_is_capturing(static_cast<hipStream_t>(stream))) {
+        if (int rc = check_operand(dst_dev, n_words * 4, "accel_dev_copy_u32", "dst")) return rc;
+        if (int rc = check_operand(src_dev, n_words * 4, "accel_dev_copy_u32", "src")) return rc;
+    }
     return copy_u32(dst_dev, src_dev, n_words, static_cast<hipStream_t>(stream));
 }
 

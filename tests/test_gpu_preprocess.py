@@ -515,6 +515,14 @@ def test_device_plumbing(gpu):
     assert np.array_equal(dst.to_numpy(np.uint32, a.shape), a)
     with pytest.raises(ValueError):
         dst.to_numpy(np.uint32, (a.size + 1,))
+    # the two kernels behind these calls get the same protection as the operator's: no launch on
+    # a host address or past the end of an allocation
+    E, L = gpu._lib, gpu.lib()
+    assert L.accel_dev_fill_u32(C.c_void_p(a.ctypes.data), 0, a.size, None) == E.ERR_ARG
+    assert L.accel_dev_fill_u32(C.c_void_p(dst.address), 0, a.size + 1, None) == E.ERR_ARG
+    assert L.accel_dev_copy_u32(C.c_void_p(dst.address), C.c_void_p(a.ctypes.data), a.size, None) == E.ERR_ARG
+    assert L.accel_dev_copy_u32(C.c_void_p(dst.address + 8), C.c_void_p(src.address), a.size, None) == E.ERR_ARG
+    assert np.array_equal(dst.to_numpy(np.uint32, a.shape), a)
     src.close()
     dst.close()
     dst.close()                                  # closing twice is harmless
