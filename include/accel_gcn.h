@@ -378,8 +378,8 @@ int accel_time_ex(accel_handle *h, const accel_run_args *args, int warmup, int i
  * of 4) are read as 16-byte vectors.  Needs no handle; asynchronous on `stream`; allocates nothing.
  * Computed on the fp32 matrix cores: sums of K products in fp32, whose order differs from a
  * sequential loop (compare against a higher-precision product, as for accel_run).  Built for
- * the shapes of a layer: many rows, K and N up to a few hundred, where the product is bound by
- * streaming X; for large K x N a BLAS is the better tool. */
+ * the shapes of a layer: many rows and N up to 128, where the product is bound by streaming
+ * X; for wider outputs (N = 256 and more) a BLAS is the better tool. */
 int accel_dense_xw(const float *X, const float *W, float *Z, int64_t rows, int32_t K, int32_t N,
                    int32_t ldx, int32_t ldz, void *stream);
 
