@@ -205,8 +205,8 @@ def gcn_layer_timing(pkg, op, g, N, K, steps, compare_rocblas=False):
     clock over `steps` launches queued back to back; a sample of rows of Z is checked against
     an fp64 product.  The dense product alone is warmed up for 80 launches: a burst of
     matrix-core work makes the GPU lower its clocks for the first 20 ms or so (launches of
-    0.48 ms grow to 0.71 ms and come back down over some thirty launches); inside the layer,
-    next to the sparse product, the same kernel takes 0.45 ms from the start."""
+    0.44 ms grow to 0.63 ms and come back down over some forty launches); inside the layer,
+    next to the sparse product, the same kernel takes 0.41 ms from the start."""
     rng = np.random.default_rng(5)
     rows = g.n_cols
     F = rng.uniform(-1, 1, (rows, K)).astype(np.float32)

@@ -84,12 +84,26 @@ __global__ __launch_bounds__(kDenseThreads, NT == 4 ? 2 : 3) void dense_xw_kerne
     // from addresses clamped into the row.  What lies past K or N is replaced by zero when the
     // registers are handed to LDS.  Rows past the end of X read the last row (their results are
     // not stored), and so does a step past the end of the walk.
+    // Each has a short form for the usual case, decided for the whole workgroup: a step that
+    // lies inside K, rows inside X, a tile inside N need no clamping, and then the addresses
+    // of a thread's loads are one base and constant strides (a few integer instructions per
+    // step instead of a hundred, which would otherwise compete with the matrix instructions
+    // for the issue slots of the SIMD).
+    constexpr int kWRowsPerLoad = kDenseThreads / kCols;      // rows of W between a thread's loads
     auto fetch_x = [&](float4 (&dst)[kDenseXLoads], const DenseStepAt &at) {
+        const int k = at.k0 + xc;
+        const int64_t r0 = at.row_block * kDenseBlockRows + (tid >> 3);
+        if (kVec && at.k0 + kDenseStep <= K && (at.row_block + 1) * kDenseBlockRows <= rows) {
+            const float *xb = X + r0 * ldx + k;
+#pragma unroll
+            for (int q = 0; q < kDenseXLoads; q++)
+                dst[q] = *reinterpret_cast<const float4 *>(xb + (int64_t)q * (kDenseThreads / 8) * ldx);
+            return;
+        }
 #pragma unroll
         for (int q = 0; q < kDenseXLoads; q++) {
-            const int64_t r = at.row_block * kDenseBlockRows + (tid >> 3) + 32 * q;
+            const int64_t r = r0 + (kDenseThreads / 8) * q;
             const float *xr = X + (r < rows ? r : rows - 1) * ldx;
-            const int k = at.k0 + xc;
             if (kVec) {
                 dst[q] = *reinterpret_cast<const float4 *>(xr + (k < K ? k : K - 4));
             } else {
@@ -102,11 +116,18 @@ __global__ __launch_bounds__(kDenseThreads, NT == 4 ? 2 : 3) void dense_xw_kerne
         }
     };
     auto fetch_w = [&](const DenseStepAt &at) {
+        const int k = at.k0 + tid / kCols, col = at.tile * kCols + tid % kCols;
+        if (at.k0 + kDenseStep <= K && (at.tile + 1) * kCols <= N) {
+            const float *wb = W + (int64_t)k * N + col;
+#pragma unroll
+            for (int i = 0; i < kWLoads; i++) wreg[i] = wb[(int64_t)i * kWRowsPerLoad * N];
+            return;
+        }
+        const int cc = col < N ? col : N - 1;
 #pragma unroll
         for (int i = 0; i < kWLoads; i++) {
-            const int e = tid + kDenseThreads * i;
-            const int k = at.k0 + e / kCols, col = at.tile * kCols + e % kCols;
-            wreg[i] = W[(int64_t)(k < K ? k : K - 1) * N + (col < N ? col : N - 1)];
+            const int ki = k + kWRowsPerLoad * i;
+            wreg[i] = W[(int64_t)(ki < K ? ki : K - 1) * N + cc];
         }
     };
 
@@ -128,19 +149,28 @@ __global__ __launch_bounds__(kDenseThreads, NT == 4 ? 2 : 3) void dense_xw_kerne
     // one step; `mine` is the half of xreg that holds its block of X
     auto step = [&](float4 (&mine)[kDenseXLoads]) {
         __syncthreads();                       // the previous step's reads of LDS are done
-        const int kx = now.k0 + xc;
+        float *xs = &x_lds[(tid >> 3) * kDenseXStride + xc];
+        float *ws = &w_lds[(tid / kCols) * kWStride + tid % kCols];
+        if (now.k0 + kDenseStep <= K && (now.tile + 1) * kCols <= N) {         // nothing to mask
 #pragma unroll
-        for (int q = 0; q < kDenseXLoads; q++) {
-            float4 x = mine[q];
-            x.x = kx < K ? x.x : 0.f; x.y = kx + 1 < K ? x.y : 0.f;
-            x.z = kx + 2 < K ? x.z : 0.f; x.w = kx + 3 < K ? x.w : 0.f;
-            *reinterpret_cast<float4 *>(&x_lds[((tid >> 3) + 32 * q) * kDenseXStride + xc]) = x;
-        }
+            for (int q = 0; q < kDenseXLoads; q++)
+                *reinterpret_cast<float4 *>(xs + q * (kDenseThreads / 8) * kDenseXStride) = mine[q];
 #pragma unroll
-        for (int i = 0; i < kWLoads; i++) {
-            const int e = tid + kDenseThreads * i;
-            const bool inside = now.k0 + e / kCols < K && now.tile * kCols + e % kCols < N;
-            w_lds[(e / kCols) * kWStride + e % kCols] = inside ? wreg[i] : 0.f;
+            for (int i = 0; i < kWLoads; i++) ws[i * kWRowsPerLoad * kWStride] = wreg[i];
+        } else {
+            const int kx = now.k0 + xc;
+            const int kw = now.k0 + tid / kCols;
+            const bool col_inside = now.tile * kCols + tid % kCols < N;
+#pragma unroll
+            for (int q = 0; q < kDenseXLoads; q++) {
+                float4 x = mine[q];
+                x.x = kx < K ? x.x : 0.f; x.y = kx + 1 < K ? x.y : 0.f;
+                x.z = kx + 2 < K ? x.z : 0.f; x.w = kx + 3 < K ? x.w : 0.f;
+                *reinterpret_cast<float4 *>(xs + q * (kDenseThreads / 8) * kDenseXStride) = x;
+            }
+#pragma unroll
+            for (int i = 0; i < kWLoads; i++)
+                ws[i * kWRowsPerLoad * kWStride] = (col_inside && kw + kWRowsPerLoad * i < K) ? wreg[i] : 0.f;
         }
         __syncthreads();
         // in flight while the matrix cores work: W of the next step, X of the one after it
