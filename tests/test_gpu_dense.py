@@ -175,3 +175,25 @@ def test_dense_product_in_a_captured_graph(gpu):
         assert so.check_dense(dZ.to_numpy(np.float32, (rows, N)), X2, W) <= so.TOL
     hip.hipGraphExecDestroy(ex); hip.hipGraphDestroy(graph); hip.hipStreamDestroy(s)
     dX.close(); dW.close(); dZ.close()
+
+
+def test_layer_and_wrapper_argument_errors(gpu):
+    g = helpers.graph_from_degrees(helpers.degree_mix(seed=5, n_long=1), seed=5)
+    op = gpu.AccelSpMM(g.indptr, g.indices, g.values, g.n_cols).preprocess()
+    W = np.ones((8, 4), np.float32)
+    with pytest.raises(gpu.AccelError):
+        gpu.GcnLayer(op, np.zeros((0, 4), np.float32))                       # empty weights
+    with pytest.raises(gpu.AccelError):
+        gpu.GcnLayer(op, W, bias=np.zeros(5, np.float32))                    # bias of the wrong length
+    layer = gpu.GcnLayer(op, W, bias=np.zeros(4, np.float32))
+    with pytest.raises(gpu.AccelError):
+        layer.forward_numpy(np.zeros((g.n_cols, 9), np.float32))             # features of the wrong width
+    with pytest.raises(gpu.AccelError):
+        gpu.dense_xw(np.zeros((4, 8), np.float32), layer._w, layer._z, 4, 8, 4)   # a host array as X
+    with pytest.raises(gpu.AccelError):
+        gpu.dense_xw(layer._z, layer._w, layer._z, 4, 8, 4, ldx=7)           # stride below K
+    with pytest.raises(gpu.AccelError):
+        gpu.dense_xw_numpy(np.zeros((4, 8), np.float32), np.zeros((7, 4), np.float32))
+    Y = layer.forward_numpy(np.zeros((g.n_cols, 8), np.float32))             # zero features: act(bias) = 0
+    assert Y.shape == (g.n_rows, 4) and not Y.any()
+    layer.close(); layer.close(); op.close()
