@@ -53,6 +53,7 @@ bool SPMM_ACCEL::preprocess()
     }
     if (rc) {
         err = accel_last_error();
+        if (err.empty()) err = meta_dir + _graph + ".block4 does not hold whole block4 entries";
         if (h) accel_destroy(h);
         h = nullptr;
         return false;
